@@ -387,8 +387,7 @@ def test_flash_attention_padding(native_ext, S, d):
 
 
 def test_flash_attention_bwd_bit_stable(native_ext):
-    """the backward kernels use no atomics: dQ / dK / dV are bit-identical call after call.  (The round-5 race of a
-    counted vmcnt wait beside LDS-DMAs is pinned structurally on the CPU: tests/test_vmcnt_audit_cpu.py.)"""
+    """the backward kernels use no atomics: dQ / dK / dV are bit-identical call after call."""
     import os
     import subprocess
     import sys
