@@ -293,8 +293,9 @@ def _load_for_inference(path, adapter=None, device=None, quant=None, fuse=True, 
             from ..quant.io import load_quantized
             m = load_quantized(path, dev)
         else:
+            from ..models.registry import load_causal_lm      # the class config.json names (Qwen3/Qwen2, Mobupel)
             bnb = BitsAndBytesConfig(load_in_4bit=True) if quant == "nf4" else None
-            m = Qwen3ForCausalLM.from_pretrained(path, dtype=torch.bfloat16, device=dev, quantization_config=bnb)
+            m = load_causal_lm(path, dtype=torch.bfloat16, device=dev, quantization_config=bnb)
     if adapter:
         from ..peft.lora import PeftModel
         m = PeftModel.from_pretrained(m, adapter)
@@ -312,6 +313,11 @@ def _add_parallel_args(p):
                    help="under torchrun: TP degree (default WORLD_SIZE / pp)")
     p.add_argument("--pipeline-parallel-size", "-pp", dest="pp", type=int, default=1,
                    help="under torchrun: pipeline stages (layers split across ranks)")
+
+
+def cmd_trace_run(a):
+    from ..infer.trace import run
+    return run(a.model, a.dtype, a.out, a.max_tokens, use_graphs=a.graphs)
 
 
 def cmd_chat(a):
@@ -1137,6 +1143,13 @@ def build_parser() -> argparse.ArgumentParser:
     p.add_argument("--load-format", dest="load_format", default="auto", choices=["auto", "safetensors", "pt"],
                    help="vLLM flag: checkpoint files are read by their extension (safetensors first)")
     p.set_defaults(fn=cmd_dl_basics)
+    p = sub.add_parser("trace-run", help="replay a token trace (JSON steps on stdin) through the engine, write logits")
+    p.add_argument("--model", required=True, help="folder with config.json + model.safetensors")
+    p.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16")
+    p.add_argument("--out", required=True, help="folder for <step>.f32 files")
+    p.add_argument("--max-tokens", type=int, default=4096, help="most tokens live requests hold at any time")
+    p.add_argument("--graphs", action="store_true", help="decode through captured hipGraphs")
+    p.set_defaults(fn=cmd_trace_run)
     p = sub.add_parser("env")
     p.set_defaults(fn=cmd_env)
 

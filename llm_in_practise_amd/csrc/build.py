@@ -6,6 +6,7 @@ project writes CDNA4 HIP directly, so the kernels are compiled by ``hipcc
 
     python -m llm_in_practise_amd.csrc.build          # both extensions, in-tree
     python -m llm_in_practise_amd.csrc.build --hip    # HIP kernels only
+    python -m llm_in_practise_amd.csrc.build --seq    # the sequence-state kernels only (_seq)
 
 Objects are cached under ``build/native`` by (source mtime, flags); compiles run in
 parallel (``MAX_JOBS``, default 8).
@@ -95,6 +96,36 @@ def build_hip_extension(jobs: int | None = None, verbose: bool = True) -> str:
     return out
 
 
+def build_seq_extension(jobs: int | None = None, verbose: bool = True) -> str:
+    """``llm_in_practise_amd._seq``: the sequence-state kernels (``kernels/seq/*.hip`` + ``seq_bindings.cpp``) as an
+    extension of their own, so a model that needs only these builds in well under a minute on a fresh checkout."""
+    inc, libs, abi = _torch_flags()
+    hipcc = os.path.join(ROCM, "bin", "hipcc")
+    kdir = os.path.join(HERE, "kernels", "seq")
+    headers = sorted(glob.glob(os.path.join(kdir, "*.h"))) + [os.path.join(HERE, "kernels", "common.h")]
+    kflags = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-ffp-contract=fast", "-Xclang", "-target-feature",
+              "-Xclang", "-packed-fp32-ops", f"-I{kdir}"]
+    bflags = ["-O2", "-std=c++17", "-fPIC", f"-D_GLIBCXX_USE_CXX11_ABI={abi}", "-D__HIP_PLATFORM_AMD__=1",
+              "-DUSE_ROCM=1", "-DTORCH_API_INCLUDE_EXTENSION_H", "-DTORCH_EXTENSION_NAME=_seq",
+              f"-I{sysconfig.get_paths()['include']}", f"-I{ROCM}/include"] + [f"-I{p}" for p in inc]
+    srcs = sorted(glob.glob(os.path.join(kdir, "*.hip")))
+    jobs = jobs or int(os.environ.get("MAX_JOBS", "8"))
+    with cf.ThreadPoolExecutor(max_workers=jobs) as ex:
+        futs = [ex.submit(_compile, s, kflags, [hipcc], headers) for s in srcs]
+        futs.append(ex.submit(_compile, os.path.join(HERE, "seq_bindings.cpp"), bflags, ["g++"], []))
+        objs = [f.result() for f in futs]
+    out = os.path.join(PKG, f"_seq{EXT_SUFFIX}")
+    tmp = f"{out}.{os.getpid()}.tmp"
+    link = [hipcc, "-shared", "-fPIC", f"--offload-arch={ARCH}", "-o", tmp] + objs
+    link += [f"-L{p}" for p in libs] + [f"-Wl,-rpath,{p}" for p in libs]
+    link += ["-lc10", "-ltorch", "-ltorch_cpu", "-ltorch_python", "-lc10_hip", "-ltorch_hip", "-lamdhip64"]
+    _run(link)
+    os.replace(tmp, out)
+    if verbose:
+        print(f"[lipa build] {os.path.relpath(out, ROOT)} ({len(srcs)} HIP sources, {ARCH})", file=sys.stderr)
+    return out
+
+
 def build_cpu_extension(verbose: bool = True):
     """Build (if needed) and import ``llm_in_practise_amd._cpu``."""
     inc, libs, abi = _torch_flags()
@@ -148,6 +179,7 @@ def main(argv=None):
     ap = argparse.ArgumentParser()
     ap.add_argument("--hip", action="store_true")
     ap.add_argument("--cpu", action="store_true")
+    ap.add_argument("--seq", action="store_true", help="the sequence-state kernels only (_seq)")
     ap.add_argument("--clean", action="store_true")
     ap.add_argument("--sanitize", choices=["address", "thread"], help="build + run the host sanitizer harness")
     a = ap.parse_args(argv)
@@ -156,7 +188,9 @@ def main(argv=None):
     if a.sanitize:
         exe = build_sanitizer_harness(a.sanitize)
         return subprocess.call([exe])
-    both = not (a.hip or a.cpu)
+    both = not (a.hip or a.cpu or a.seq)
+    if a.seq or both:
+        build_seq_extension()
     if a.hip or both:
         build_hip_extension()
     if a.cpu or both:

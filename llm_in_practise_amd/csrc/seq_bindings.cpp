@@ -1,0 +1,322 @@
+// PyTorch bindings of the sequence-state kernels (csrc/kernels/seq/*.hip): raw pointers + the current HIP stream,
+// so every op is ordered with PyTorch's own work and can be captured in a hipGraph.  Shapes and bounds that the
+// kernels assume are checked here, on the host, before anything is launched.
+#include <torch/extension.h>
+#include <ATen/hip/HIPContext.h>
+#include <hip/hip_runtime.h>
+
+#include <vector>
+
+struct SeqDesc {
+  const int* seq_off;
+  const int* slots;
+  const int* pos0;
+  const int* tok_seq;
+  const int* tok_pos;
+  const int* live;
+  int B, Ttot;
+};
+
+void seq_embed_sincos(int, const long*, const int*, const void*, const float*, float*, int, int, float, hipStream_t);
+void seq_rms_f32(int, const float*, const float*, void*, int, int, float, hipStream_t);
+void seq_gated_residual(int, float*, const void*, int, const void*, int, const float*, const float*, const float*,
+                        void*, int, int, float, hipStream_t);
+void seq_dual_norm_mean(int, const void*, const void*, const float*, const float*, void*, int, int, float, hipStream_t);
+void seq_polynorm(int, const void*, const float*, void*, int, int, float, hipStream_t);
+void seq_head_norm_gate(int, const float*, const float*, int, const void*, int, void*, int, int, int, float,
+                        hipStream_t);
+void seq_decay_gate(const float*, const float*, const float*, float*, int, int, int, hipStream_t);
+void seq_short_conv(int, int, const void*, int, const float*, void*, void*, int, int, int, const int*,
+                    const float* const*, const float*, SeqDesc, float, hipStream_t);
+void seq_mlstm_scan(int, const void*, int, const void*, int, const void*, int, const float*, const float*, const float*,
+                    const float*, float, float, float*, float*, float*, float*, int, int, int, SeqDesc, hipStream_t);
+void seq_delta_scan(int, const void*, int, const void*, int, const void*, int, const float*, const float*, float*,
+                    float*, int, int, int, int, SeqDesc, hipStream_t);
+void seq_talk_attention(int, const void*, int, const void*, const void*, float*, float*, float*, const float*,
+                        const void*, int, void*, int, int, int, int, int, int, float, SeqDesc, hipStream_t);
+int seq_scan_max_dk();
+int seq_conv_max_head();
+int seq_conv_max_taps();
+int seq_attn_max_cols();
+
+using at::Tensor;
+using c10::optional;
+
+static hipStream_t stream() { return at::hip::getCurrentHIPStream().stream(); }
+
+static int code_of(const Tensor& t) {
+  TORCH_CHECK(t.scalar_type() == at::kBFloat16 || t.scalar_type() == at::kFloat, "activations must be bf16 or float");
+  return t.scalar_type() == at::kBFloat16 ? 0 : 1;
+}
+static void f32c(const Tensor& t, const char* n) {
+  TORCH_CHECK(t.is_cuda() && t.scalar_type() == at::kFloat && t.is_contiguous(), n, ": float, contiguous, on the GPU");
+}
+static void rows(const Tensor& t, int64_t T, int64_t C, int code, const char* n) {   // [T, C] view, unit inner stride
+  TORCH_CHECK(t.is_cuda() && t.dim() == 2 && t.size(0) == T && t.size(1) == C && (T == 0 || t.stride(1) == 1) &&
+                  code_of(t) == code, n, ": wrong shape, stride or dtype");
+}
+static int ld(const Tensor& t) { return (int)t.stride(0); }
+
+// desc = [seq_off(B+1), slots(B), pos0(B), tok_seq(T), tok_pos(T)] int32 on the GPU, live optional [B]
+static SeqDesc desc_of(const std::vector<Tensor>& d, const optional<Tensor>& live, int64_t T) {
+  TORCH_CHECK(d.size() == 5, "sequence descriptor: 5 tensors");
+  for (auto& t : d) TORCH_CHECK(t.is_cuda() && t.scalar_type() == at::kInt && t.is_contiguous(), "descriptor: int32");
+  const int B = (int)d[1].numel();
+  TORCH_CHECK(d[0].numel() == B + 1 && d[2].numel() == B && d[3].numel() == T && d[4].numel() == T,
+              "descriptor sizes do not fit the token count");
+  SeqDesc s{d[0].data_ptr<int>(), d[1].data_ptr<int>(), d[2].data_ptr<int>(), d[3].data_ptr<int>(),
+            d[4].data_ptr<int>(), nullptr, B, (int)T};
+  if (live && live->defined()) {
+    TORCH_CHECK(live->is_cuda() && live->scalar_type() == at::kInt && live->numel() >= B, "live: int32 [B]");
+    s.live = live->data_ptr<int>();
+  }
+  return s;
+}
+
+Tensor embed_sincos(Tensor tok, Tensor pos, Tensor table, Tensor inv_freq, double scale) {
+  TORCH_CHECK(tok.is_cuda() && tok.scalar_type() == at::kLong && tok.is_contiguous(), "tokens: int64");
+  TORCH_CHECK(pos.is_cuda() && pos.scalar_type() == at::kInt && pos.is_contiguous() && pos.numel() == tok.numel(),
+              "positions: int32, one per token");
+  TORCH_CHECK(table.is_cuda() && table.is_contiguous() && table.dim() == 2, "table");
+  const int T = (int)tok.numel(), W = (int)table.size(1);
+  f32c(inv_freq, "inv_freq");
+  TORCH_CHECK(inv_freq.numel() * 2 >= W, "inv_freq too short");
+  auto x = at::empty({T, W}, table.options().dtype(at::kFloat));
+  seq_embed_sincos(code_of(table), tok.data_ptr<long>(), pos.data_ptr<int>(), table.data_ptr(),
+                   inv_freq.data_ptr<float>(), x.data_ptr<float>(), T, W, (float)scale, stream());
+  return x;
+}
+
+Tensor rms_f32(Tensor x, Tensor w, double eps, bool out_bf16) {
+  f32c(x, "x");
+  f32c(w, "w");
+  const int W = (int)x.size(-1), T = (int)(x.numel() / W);
+  TORCH_CHECK(w.numel() == W, "norm weight size");
+  auto out = at::empty_like(x, x.options().dtype(out_bf16 ? at::kBFloat16 : at::kFloat));
+  seq_rms_f32(out_bf16 ? 0 : 1, x.data_ptr<float>(), w.data_ptr<float>(), out.data_ptr(), T, W, (float)eps, stream());
+  return out;
+}
+
+// x (float, in place) += norm(y * sigmoid(r + b)) * wb; returns norm(x) * wn in y's dtype when wn is given
+optional<Tensor> gated_residual(Tensor x, Tensor y, Tensor r, Tensor b, Tensor wb, optional<Tensor> wn, double eps) {
+  f32c(x, "x");
+  const int W = (int)x.size(-1), T = (int)(x.numel() / W), code = code_of(y);
+  rows(y, T, W, code, "y");
+  rows(r, T, W, code, "r");
+  f32c(b, "b");
+  f32c(wb, "wb");
+  TORCH_CHECK(b.numel() == W && wb.numel() == W, "gate bias / norm weight size");
+  optional<Tensor> h;
+  const float* wnp = nullptr;
+  void* hp = nullptr;
+  if (wn && wn->defined()) {
+    f32c(*wn, "wn");
+    TORCH_CHECK(wn->numel() == W, "next norm weight size");
+    h = at::empty({T, W}, y.options());
+    wnp = wn->data_ptr<float>();
+    hp = h->data_ptr();
+  }
+  seq_gated_residual(code, x.data_ptr<float>(), y.data_ptr(), ld(y), r.data_ptr(), ld(r), b.data_ptr<float>(),
+                     wb.data_ptr<float>(), wnp, hp, T, W, (float)eps, stream());
+  return h;
+}
+
+Tensor dual_norm_mean(Tensor a, Tensor b, Tensor wa, Tensor wb, double eps) {
+  const int code = code_of(a);
+  TORCH_CHECK(a.is_cuda() && a.is_contiguous() && b.is_contiguous() && a.sizes() == b.sizes() && code_of(b) == code,
+              "branches must match");
+  const int W = (int)a.size(-1), T = (int)(a.numel() / W);
+  f32c(wa, "wa");
+  f32c(wb, "wb");
+  TORCH_CHECK(wa.numel() == W && wb.numel() == W, "norm weight size");
+  auto out = at::empty_like(a);
+  seq_dual_norm_mean(code, a.data_ptr(), b.data_ptr(), wa.data_ptr<float>(), wb.data_ptr<float>(), out.data_ptr(), T, W,
+                     (float)eps, stream());
+  return out;
+}
+
+Tensor polynorm(Tensor z, Tensor coef, double eps) {
+  TORCH_CHECK(z.is_cuda() && z.is_contiguous(), "z");
+  f32c(coef, "coef");
+  TORCH_CHECK(coef.numel() == 4, "PolyNorm has four coefficients");
+  const int F = (int)z.size(-1), T = (int)(z.numel() / F);
+  auto out = at::empty_like(z);
+  seq_polynorm(code_of(z), z.data_ptr(), coef.data_ptr<float>(), out.data_ptr(), T, F, (float)eps, stream());
+  return out;
+}
+
+Tensor head_norm_gate(Tensor o, Tensor w, Tensor gate, double eps) {
+  f32c(o, "o");
+  TORCH_CHECK(o.dim() == 3, "o: [T, H, dv]");
+  const int T = (int)o.size(0), H = (int)o.size(1), dv = (int)o.size(2), code = code_of(gate);
+  f32c(w, "w");
+  TORCH_CHECK(w.numel() == dv || w.numel() == (int64_t)H * dv, "norm weight: [dv] or [H * dv]");
+  rows(gate, T, (int64_t)H * dv, code, "gate");
+  auto out = at::empty({T, (int64_t)H * dv}, gate.options());
+  seq_head_norm_gate(code, o.data_ptr<float>(), w.data_ptr<float>(), w.numel() != dv, gate.data_ptr(), ld(gate),
+                     out.data_ptr(), T, H, dv, (float)eps, stream());
+  return out;
+}
+
+Tensor decay_gate(Tensor pre, Tensor bias, Tensor a_log, int64_t dk) {
+  f32c(pre, "pre");
+  f32c(bias, "bias");
+  f32c(a_log, "A_log");
+  const int HD = (int)pre.size(-1), T = (int)(pre.numel() / HD);
+  TORCH_CHECK(bias.numel() == HD && HD % dk == 0 && a_log.numel() == HD / dk, "decay gate sizes");
+  auto g = at::empty_like(pre);
+  seq_decay_gate(pre.data_ptr<float>(), bias.data_ptr<float>(), a_log.data_ptr<float>(), g.data_ptr<float>(), T, HD,
+                 (int)dk, stream());
+  return g;
+}
+
+// u [T, C] (a column slice of a GEMM output is fine), w float [C, taps], state [slots, taps-1, C] in u's dtype
+// (updated in place), segs = [[c0, heads, head width, mode]...], seg_w / seg_scale per segment.
+Tensor short_conv(Tensor u, Tensor w, optional<Tensor> state, std::vector<std::vector<int64_t>> segs,
+                  std::vector<optional<Tensor>> seg_w, std::vector<double> seg_scale, std::vector<Tensor> desc,
+                  optional<Tensor> live, double eps, bool out_f32) {
+  const int code = code_of(u);
+  TORCH_CHECK(u.dim() == 2, "u: [T, C]");
+  const int64_t T = u.size(0), C = u.size(1);
+  rows(u, T, C, code, "u");
+  f32c(w, "conv weight");
+  TORCH_CHECK(w.dim() == 2 && w.size(0) == C, "conv weight: [C, taps]");
+  const int taps = (int)w.size(1);
+  TORCH_CHECK(taps >= 1 && taps <= seq_conv_max_taps(), "conv taps out of range");
+  SeqDesc d = desc_of(desc, live, T);
+  void* sp = nullptr;
+  if (taps > 1) {
+    TORCH_CHECK(state && state->defined() && state->is_cuda() && state->is_contiguous() && state->dim() == 3 &&
+                    state->size(1) == taps - 1 && state->size(2) == C && code_of(*state) == code,
+                "conv state: [slots, taps-1, C] in the input's dtype");
+    sp = state->data_ptr();
+  }
+  const int nseg = (int)segs.size();
+  TORCH_CHECK(nseg >= 1 && nseg <= 3 && (int)seg_w.size() == nseg && (int)seg_scale.size() == nseg, "1-3 segments");
+  int flat[12];
+  const float* wp[3];
+  float sc[3];
+  int64_t c = 0;
+  for (int i = 0; i < nseg; ++i) {
+    TORCH_CHECK(segs[i].size() == 4 && segs[i][0] == c && segs[i][2] >= 1 && segs[i][2] <= seq_conv_max_head(),
+                "segments must tile the channels; head width <= ", seq_conv_max_head());
+    for (int j = 0; j < 4; ++j) flat[4 * i + j] = (int)segs[i][j];
+    c += segs[i][1] * segs[i][2];
+    wp[i] = nullptr;
+    if (segs[i][3] == 1) {
+      TORCH_CHECK(seg_w[i] && seg_w[i]->defined(), "mode 1 needs a norm weight");
+      f32c(*seg_w[i], "segment norm weight");
+      TORCH_CHECK(seg_w[i]->numel() == segs[i][2], "segment norm weight size");
+      wp[i] = seg_w[i]->data_ptr<float>();
+    }
+    sc[i] = (float)seg_scale[i];
+  }
+  TORCH_CHECK(c == C, "segments must cover all channels");
+  auto out = at::empty({T, C}, u.options().dtype(out_f32 ? at::kFloat : u.scalar_type()));
+  seq_short_conv(code, out_f32 ? 1 : 0, u.data_ptr(), ld(u), w.data_ptr<float>(), sp, out.data_ptr(), (int)C, taps, nseg,
+                 flat, wp, sc, d, (float)eps, stream());
+  return out;
+}
+
+static void check_state(const Tensor& S, int64_t H, int64_t dv, int64_t dk) {
+  f32c(S, "state");
+  TORCH_CHECK(S.dim() == 4 && S.size(1) == H && S.size(2) == dv && S.size(3) == dk, "state: [slots, H, dv, dk]");
+}
+
+Tensor mlstm_scan(Tensor q, Tensor k, Tensor v, Tensor ipre, Tensor fpre, Tensor ib, Tensor fb, double cap,
+                  double qscale, Tensor S, Tensor N, Tensor M, int64_t H, std::vector<Tensor> desc,
+                  optional<Tensor> live) {
+  const int code = code_of(q);
+  const int64_t T = q.size(0);
+  TORCH_CHECK(q.dim() == 2 && q.size(1) % H == 0 && v.dim() == 2 && v.size(1) % H == 0, "q/k/v: [T, H * d]");
+  const int64_t dk = q.size(1) / H, dv = v.size(1) / H;
+  rows(q, T, H * dk, code, "q");
+  rows(k, T, H * dk, code, "k");
+  rows(v, T, H * dv, code, "v");
+  f32c(ipre, "ipre");
+  f32c(fpre, "fpre");
+  f32c(ib, "ib");
+  f32c(fb, "fb");
+  TORCH_CHECK(ipre.numel() == T * H && fpre.numel() == T * H && ib.numel() == H && fb.numel() == H, "gate sizes");
+  TORCH_CHECK(dk <= seq_scan_max_dk(), "mlstm: key size above ", seq_scan_max_dk());
+  TORCH_CHECK(cap > 0, "gate cap must be positive");
+  check_state(S, H, dv, dk);
+  f32c(N, "n");
+  f32c(M, "m");
+  TORCH_CHECK(N.numel() == S.size(0) * H * dk && M.numel() == S.size(0) * H, "n / m state sizes");
+  SeqDesc d = desc_of(desc, live, T);
+  auto out = at::empty({T, H, dv}, S.options());
+  seq_mlstm_scan(code, q.data_ptr(), ld(q), k.data_ptr(), ld(k), v.data_ptr(), ld(v), ipre.data_ptr<float>(),
+                 fpre.data_ptr<float>(), ib.data_ptr<float>(), fb.data_ptr<float>(), (float)cap, (float)qscale,
+                 S.data_ptr<float>(), N.data_ptr<float>(), M.data_ptr<float>(), out.data_ptr<float>(), (int)H, (int)dk,
+                 (int)dv, d, stream());
+  return out;
+}
+
+Tensor delta_scan(Tensor q, Tensor k, Tensor v, Tensor g, Tensor bpre, Tensor S, int64_t H, int64_t G,
+                  std::vector<Tensor> desc, optional<Tensor> live) {
+  const int code = code_of(q);
+  const int64_t T = q.size(0);
+  TORCH_CHECK(G >= 1 && H % G == 0 && q.dim() == 2 && q.size(1) % G == 0 && v.dim() == 2 && v.size(1) % H == 0,
+              "q/k: [T, G * dk], v: [T, H * dv]");
+  const int64_t dk = q.size(1) / G, dv = v.size(1) / H;
+  rows(q, T, G * dk, code, "q");
+  rows(k, T, G * dk, code, "k");
+  rows(v, T, H * dv, code, "v");
+  f32c(g, "g");
+  f32c(bpre, "bpre");
+  TORCH_CHECK(g.numel() == T * H * dk && bpre.numel() == T * H, "decay / beta sizes");
+  TORCH_CHECK(dk <= seq_scan_max_dk(), "delta rule: key size above ", seq_scan_max_dk());
+  check_state(S, H, dv, dk);
+  SeqDesc d = desc_of(desc, live, T);
+  auto out = at::empty({T, H, dv}, S.options());
+  seq_delta_scan(code, q.data_ptr(), ld(q), k.data_ptr(), ld(k), v.data_ptr(), ld(v), g.data_ptr<float>(),
+                 bpre.data_ptr<float>(), S.data_ptr<float>(), out.data_ptr<float>(), (int)H, (int)G, (int)dk, (int)dv, d,
+                 stream());
+  return out;
+}
+
+// q [T, H*dk]; kc [slots, max_len, G*dk], vc [slots, max_len, G*dv] already hold this step's keys and values
+Tensor talk_attention(Tensor q, Tensor kc, Tensor vc, Tensor talk, Tensor gate, int64_t H, int64_t G, double scale,
+                      int64_t nsplit, std::vector<Tensor> desc) {
+  const int code = code_of(q);
+  const int64_t T = q.size(0);
+  TORCH_CHECK(G >= 1 && H % G == 0 && q.dim() == 2 && q.size(1) % H == 0, "q: [T, H * dk]");
+  const int64_t dk = q.size(1) / H;
+  rows(q, T, H * dk, code, "q");
+  TORCH_CHECK(kc.is_cuda() && kc.is_contiguous() && kc.dim() == 3 && kc.size(2) == G * dk && code_of(kc) == code,
+              "key cache: [slots, max_len, G * dk]");
+  TORCH_CHECK(vc.is_cuda() && vc.is_contiguous() && vc.dim() == 3 && vc.size(0) == kc.size(0) &&
+                  vc.size(1) == kc.size(1) && vc.size(2) % G == 0 && code_of(vc) == code,
+              "value cache: [slots, max_len, G * dv]");
+  const int64_t dv = vc.size(2) / G, max_len = kc.size(1);
+  TORCH_CHECK(G * dv <= seq_attn_max_cols(), "attention: G * dv above ", seq_attn_max_cols());
+  TORCH_CHECK(nsplit >= 1 && nsplit <= 1024, "nsplit");
+  f32c(talk, "talk");
+  TORCH_CHECK(talk.numel() == H * H, "talk: [H, H]");
+  rows(gate, T, H * dv, code, "gate");
+  SeqDesc d = desc_of(desc, optional<Tensor>(), T);
+  auto fo = q.options().dtype(at::kFloat);
+  auto pm = at::empty({T, H, nsplit}, fo), pl = at::empty({T, H, nsplit}, fo);
+  auto pu = at::empty({T, H, nsplit, G * dv}, fo);
+  auto out = at::empty({T, H * dv}, q.options());
+  seq_talk_attention(code, q.data_ptr(), ld(q), kc.data_ptr(), vc.data_ptr(), pm.data_ptr<float>(),
+                     pl.data_ptr<float>(), pu.data_ptr<float>(), talk.data_ptr<float>(), gate.data_ptr(), ld(gate),
+                     out.data_ptr(), (int)H, (int)G, (int)dk, (int)dv, (int)max_len, (int)nsplit, (float)scale, d,
+                     stream());
+  return out;
+}
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
+  m.def("embed_sincos", &embed_sincos);
+  m.def("rms_f32", &rms_f32);
+  m.def("gated_residual", &gated_residual);
+  m.def("dual_norm_mean", &dual_norm_mean);
+  m.def("polynorm", &polynorm);
+  m.def("head_norm_gate", &head_norm_gate);
+  m.def("decay_gate", &decay_gate);
+  m.def("short_conv", &short_conv);
+  m.def("mlstm_scan", &mlstm_scan);
+  m.def("delta_scan", &delta_scan);
+  m.def("talk_attention", &talk_attention);
+}

@@ -31,7 +31,7 @@ from typing import Any
 
 import torch
 
-from ..models.common import KVCache, PackedPrefill
+from ..models.common import KVCache
 from ..ops.decode import sample
 from ..ops.linear import head_logits
 from ..train.data import render_chatml
@@ -351,7 +351,7 @@ class ServingEngine:
                  use_graphs: bool | None = None, tp_group=None, prefix_cache_blocks: int = 0,
                  prefix_block: int = 64, chunked_prefill: int = 0, lora_modules: dict[str, str] | None = None,
                  host_cache_blocks: int = 0, kv_remote_url: str | None = None,
-                 gpu_memory_utilization: float | None = None):
+                 gpu_memory_utilization: float | None = None, start: bool = True):
         """``tp_group``: the model was sharded by ``parallel.tensor_parallel`` over this group.
         The engine then runs SPMD — group rank 0 owns the request queue and broadcasts each
         iteration's admissions; the other ranks call :meth:`follower_loop` and replay exactly the
@@ -404,19 +404,33 @@ class ServingEngine:
         self.h_latency = _Histogram([0.05, 0.1, 0.25, 0.5, 1, 2, 5, 10, 30, 60])
         self.h_ttft = _Histogram([0.01, 0.025, 0.05, 0.1, 0.2, 0.5, 1, 2, 5])
         self.queue_time_ewma: float | None = None
+        # models whose sequences hold more than K/V rows (recurrent state, convolution inputs) bring their own slot
+        # pool (models/common.py SeqStateCache); it answers the same view calls as KVCache
+        self.stateful = hasattr(self.lm, "make_cache")
+        self._head = getattr(self.lm, "compute_logits", None) or (lambda h: head_logits(h, self.lm.lm_head.weight))
+        if self.stateful and (prefix_cache_blocks > 0 or lora_modules or tp_group is not None):
+            raise ValueError("prefix caching, LoRA modules and tensor parallelism need a plain K/V model: a recurrent "
+                             "state cannot be rebuilt from cached K/V chunks")
         if gpu_memory_utilization is not None and self.device.type == "cuda":
             # the KV pool sized from the memory fraction (vLLM --gpu-memory-utilization), capped by max_batch
             elt = torch.finfo(self.lm.lm_head.weight.dtype).bits // 8
-            slot = 2 * cfg.num_hidden_layers * self.max_len * cfg.num_key_value_heads * cfg.head_dim * elt
+            if self.stateful:
+                from ..models.common import SeqStateCache
+                slot = SeqStateCache.slot_bytes(self.lm.model.state_specs(), self.max_len, self.lm.lm_head.weight.dtype)
+            else:
+                slot = 2 * cfg.num_hidden_layers * self.max_len * cfg.num_key_value_heads * cfg.head_dim * elt
             reserve = (2 << 30) + prefill_token_budget * (16 * cfg.hidden_size + 6 * getattr(cfg, "intermediate_size", 0))
             fit = kv_slots_for_budget(torch.cuda.get_device_properties(self.device).total_memory,
                                       torch.cuda.memory_allocated(self.device), gpu_memory_utilization, slot, reserve)
             max_batch = max(1, min(max_batch, fit))
             self.max_batch = max_batch
             self.max_prefill_batch = min(self.max_prefill_batch, max_batch)
-        self.cache = KVCache(cfg.num_hidden_layers, max_batch, self.max_len, cfg.num_key_value_heads, cfg.head_dim,
-                             self.lm.lm_head.weight.dtype, self.device)
-        self.cache.pos = torch.zeros(max_batch, dtype=torch.long, device=self.device)
+        if self.stateful:
+            self.cache = self.lm.make_cache(max_batch, self.max_len, self.device)
+        else:
+            self.cache = KVCache(cfg.num_hidden_layers, max_batch, self.max_len, cfg.num_key_value_heads, cfg.head_dim,
+                                 self.lm.lm_head.weight.dtype, self.device)
+            self.cache.pos = torch.zeros(max_batch, dtype=torch.long, device=self.device)
         self.prefix = None
         remote = None
         if kv_remote_url and prefix_cache_blocks > 0:
@@ -456,7 +470,7 @@ class ServingEngine:
         self._stop = False
         self._closing = False
         self._worker = None
-        if self.tp_rank == 0:
+        if self.tp_rank == 0 and start:    # start=False: the caller drives forward_prefill / forward_decode itself
             self._worker = threading.Thread(target=self._loop, daemon=True)
             self._worker.start()
 
@@ -692,13 +706,9 @@ class ServingEngine:
         if self.mlora is not None:
             self.mlora.use_rows(None)
 
-    def _slot_view(self, slot: int, length: int) -> KVCache:
-        view = KVCache.__new__(KVCache)
-        view.k = [t[slot:slot + 1] for t in self.cache.k]
-        view.v = [t[slot:slot + 1] for t in self.cache.v]
-        view.len, view.max_len, view.batch, view.pos = length, self.cache.max_len, 1, None
-        view._rows = self.cache._rows[:1]
-        return view
+    def _slot_view(self, slot: int, length: int, n: int = 0):
+        """``n`` more tokens for the sequence of ``slot``, which holds ``length`` already."""
+        return self.cache.slot_view(slot, length, n)
 
     def _prefill_chunks(self):
         """One chunk of at most ``chunked_prefill`` prompt tokens (oldest prefilling slot first)
@@ -716,7 +726,7 @@ class ServingEngine:
         ids = torch.tensor([r.prompt_ids[P:P + C]], dtype=torch.long, device=self.device)
         self._rows_for([(r.adapter, C)])
         try:
-            h = self.lm.model(ids, None, self._slot_view(slot, P), None)
+            h = self.lm.model(ids, None, self._slot_view(slot, P, C), None)
         finally:
             self._rows_done()
         s.prefilled = P + C
@@ -726,7 +736,7 @@ class ServingEngine:
             return
         s.prefilled = -1
         self.stats["prompt_tokens_total"] += L
-        logits = head_logits(h[-1:], self.lm.lm_head.weight)
+        logits = self._head(h[-1:])
         dev_toks, toks = self._sample(logits, [slot])
         self.next_tok[slot] = dev_toks[0]
         if self.prefix is not None:
@@ -737,14 +747,14 @@ class ServingEngine:
         lm = self.lm
         P = len(idx) * self.prefix.block
         self.prefix.load(idx, self.cache, slot)
-        view = self._slot_view(slot, P)
+        view = self._slot_view(slot, P, len(r.prompt_ids) - P)
         ids = torch.tensor([r.prompt_ids[P:]], dtype=torch.long, device=self.device)
         self._rows_for([(r.adapter, len(r.prompt_ids) - P)])
         try:
             h = lm.model(ids, None, view, None)
         finally:
             self._rows_done()
-        logits = head_logits(h[-1:], lm.lm_head.weight)
+        logits = self._head(h[-1:])
         L = len(r.prompt_ids)
         self.cache.pos[slot] = L
         self.slots[slot] = _Slot(r)
@@ -754,30 +764,38 @@ class ServingEngine:
         self._accept(slot, toks[0], time.time())
         self.stats["batches_total"] += 1
 
+    def forward_prefill(self, new):
+        """The prefill forward of one admission: the prompts of ``new`` = [(slot, request)] packed back to back (no
+        padding) straight into their cache slots.  Returns the hidden states of all packed tokens and the packed
+        view (``.last``: each prompt's last row; for replaying given tokens, any row can be read).  The slots'
+        positions stand at their prompt lengths afterwards."""
+        lens = [len(r.prompt_ids) for _, r in new]
+        ids = torch.tensor([[t for _, r in new for t in r.prompt_ids]], dtype=torch.long).to(self.device)
+        pp = self.cache.packed([s for s, _ in new], lens, self.device)
+        self._rows_for([(r.adapter, n) for (_, r), n in zip(new, lens)])
+        try:
+            h = self.lm.model(ids, pp.positions, pp, None)
+        finally:
+            self._rows_done()
+        rows = torch.tensor([s for s, _ in new], device=self.device)
+        self.cache.pos[rows] = torch.tensor(lens, dtype=self.cache.pos.dtype, device=self.device)
+        for slot, r in new:
+            self.slots[slot] = _Slot(r)
+            self.stats["prompt_tokens_total"] += len(r.prompt_ids)
+        self.stats["batches_total"] += 1
+        return h, pp
+
     def _admit_batch(self, new):
         """Prefill the admitted prompts packed back to back (no padding) directly into their
         cache slots (models/common.py ``PackedPrefill``), sample each one's first token."""
-        lm = self.lm
-        lens = [len(r.prompt_ids) for _, r in new]
-        ids = torch.tensor([[t for _, r in new for t in r.prompt_ids]], dtype=torch.long).to(self.device)
-        pp = PackedPrefill(self.cache, [s for s, _ in new], lens, self.device)
-        self._rows_for([(r.adapter, n) for (_, r), n in zip(new, lens)])
-        try:
-            h = lm.model(ids, pp.positions, pp, None)
-        finally:
-            self._rows_done()
-        logits = head_logits(h[pp.last], lm.lm_head.weight)
+        h, pp = self.forward_prefill(new)
+        logits = self._head(h[pp.last])
         rows = torch.tensor([s for s, _ in new], device=self.device)
-        self.cache.pos[rows] = torch.tensor(lens, dtype=torch.long, device=self.device)
         now = time.time()
-        for b, (slot, r) in enumerate(new):
-            self.slots[slot] = _Slot(r)
-            self.stats["prompt_tokens_total"] += len(r.prompt_ids)
         dev_toks, toks = self._sample(logits, [s for s, _ in new])
         self.next_tok[rows] = dev_toks
         for b, (slot, r) in enumerate(new):
             self._accept(slot, toks[b], now)
-        self.stats["batches_total"] += 1
 
     def _sample(self, logits, slot_ids):
         """Sample one token per row, grouping rows with identical sampling parameters.
@@ -859,17 +877,21 @@ class ServingEngine:
         self.slots[slot] = None
         self.cache.pos[slot] = 0
 
-    def _decode_step(self):
+    def forward_decode(self, active: list[int]):
+        """One decode step for the slots ``active`` (their next input tokens stand in ``self.next_tok``): rows
+        ``[0, max(active)]`` run — through the captured graph of their bucket when graphs are on — and every active
+        row appends at its own position.  Returns the logits of the active rows, in their order."""
         lm = self.lm
-        active = [i for i, s in enumerate(self.slots) if s is not None and s.prefilled < 0]
-        self.stats["running"] = len(active)
         n = active[-1] + 1                       # slots fill lowest-first: decode rows [0, n) only
         if self.graphs is not None:              # hipGraph replay of the whole step (bucket >= n rows)
             n = self.graphs.bucket(n)
+        if self.stateful:                        # rows that are idle or mid chunked prefill keep their state
+            self.cache.set_live(active, n)
+        if self.graphs is not None:
             logits = self.graphs.step(None, n)
         else:
             h = lm.model(self.next_tok[:n, None], None, self.cache.head_rows(n), None)   # per-row positions
-            logits = head_logits(h, lm.lm_head.weight)
+            logits = self._head(h)
         free = [i for i in range(n) if self.slots[i] is None]
         if free:                                                              # idle rows stay at position 0
             self.cache.pos[torch.tensor(free, device=self.device)] = 0
@@ -877,9 +899,21 @@ class ServingEngine:
             s = self.slots[i]     # (the next chunk overwrites it): put its position back
             if s is not None and s.prefilled >= 0:
                 self.cache.pos[i] = s.prefilled
-        rows = torch.tensor(active, device=self.device)
         if len(active) != n:
-            logits = logits[rows]
+            logits = logits[torch.tensor(active, device=self.device)]
+        self.stats["decode_steps_total"] += 1
+        return logits
+
+    def release(self, slot: int):
+        """Give a slot back: its rows and state are reused by the next sequence that starts there."""
+        self.slots[slot] = None
+        self.cache.pos[slot] = 0
+
+    def _decode_step(self):
+        active = [i for i, s in enumerate(self.slots) if s is not None and s.prefilled < 0]
+        self.stats["running"] = len(active)
+        logits = self.forward_decode(active)
+        rows = torch.tensor(active, device=self.device)
         if self.pipeline and all(self.slots[s].req.params.repetition_penalty == 1.0 for s in active):
             # asynchronous: the sampled tokens stay on the device (next step's input), a pinned
             # copy + event hand them to the host, and the host accepts the PREVIOUS step's
@@ -901,7 +935,6 @@ class ServingEngine:
             now = time.time()
             for j, slot in enumerate(active):
                 self._accept(slot, toks[j], now)
-        self.stats["decode_steps_total"] += 1
         self.stats["running"] = sum(s is not None for s in self.slots)
 
     def _process_pending(self, pend):

@@ -79,9 +79,12 @@ def generate(model, input_ids: torch.Tensor, attention_mask: torch.Tensor | None
         attention_mask = torch.ones_like(input_ids)
     lens = attention_mask.long().sum(1)
     mcfg = lm.config
-    n_layers = mcfg.num_hidden_layers
-    hkv, d = mcfg.num_key_value_heads, mcfg.head_dim
-    cache = KVCache(n_layers, B, S + cfg.max_new_tokens, hkv, d, lm.lm_head.weight.dtype, dev)
+    if hasattr(lm, "make_cache"):       # models with per-sequence state beyond K/V bring their own slot pool
+        cache = lm.make_cache(B, S + cfg.max_new_tokens, dev)
+    else:
+        cache = KVCache(mcfg.num_hidden_layers, B, S + cfg.max_new_tokens, mcfg.num_key_value_heads, mcfg.head_dim,
+                        lm.lm_head.weight.dtype, dev)
+    head = getattr(lm, "compute_logits", None) or (lambda x: x @ lm.lm_head.weight.t())
     temperature = cfg.temperature if cfg.do_sample else 0.0
     if cfg.seed is not None:
         from ..ops.decode import seed_sampler
@@ -94,7 +97,7 @@ def generate(model, input_ids: torch.Tensor, attention_mask: torch.Tensor | None
     kv_lens = lens.to(torch.int32)
     h = lm.model(input_ids, None, cache, kv_lens)                     # [B*S, H]
     last = h.view(B, S, -1)[torch.arange(B, device=dev), lens - 1]   # [B, H]
-    logits = last @ lm.lm_head.weight.t()
+    logits = head(last)
     history = torch.full((B, S + cfg.max_new_tokens), -1, dtype=torch.int32, device=dev)
     history[:, :S] = torch.where(attention_mask.bool(), input_ids, torch.full_like(input_ids, -1)).to(torch.int32)
     cache.start_decode(lens)
@@ -117,7 +120,7 @@ def generate(model, input_ids: torch.Tensor, attention_mask: torch.Tensor | None
         if t + 1 == cfg.max_new_tokens:
             break
         hd = lm.model(tok[:, None], None, cache, None)                # decode step: [B, H]
-        logits = hd @ lm.lm_head.weight.t()
+        logits = head(hd)
     if streamer is not None:
         streamer.end()
     if was_training:

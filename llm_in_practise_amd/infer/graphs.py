@@ -41,7 +41,7 @@ class DecodeGraphs:
         self.lm, self.cache = lm, cache
         self.max_batch = max_batch or cache.batch
         self.buckets = buckets or _buckets(self.max_batch)
-        dev = cache.k[0].device
+        dev = cache.pos.device
         self.tokens = tokens if tokens is not None else torch.zeros(self.max_batch, dtype=torch.long, device=dev)
         self.graphs: dict[int, torch.cuda.CUDAGraph] = {}
         self.logits: dict[int, torch.Tensor] = {}
@@ -50,7 +50,8 @@ class DecodeGraphs:
 
     def _forward(self, n: int) -> torch.Tensor:
         h = self.lm.model(self.tokens[:n, None], None, self.cache.head_rows(n), None)
-        return head_logits(h, self.lm.lm_head.weight)
+        head = getattr(self.lm, "compute_logits", None)
+        return head(h) if head is not None else head_logits(h, self.lm.lm_head.weight)
 
     @torch.no_grad()
     def _capture_all(self):

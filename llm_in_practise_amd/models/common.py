@@ -259,8 +259,135 @@ class KVCache:
         v._rows = self._rows[:n]
         return v
 
+    def packed(self, slots: list[int], lens: list[int], device=None) -> "PackedPrefill":
+        """Prompts packed back to back, prefilled straight into ``slots`` (the engine's admission path)."""
+        return PackedPrefill(self, slots, lens, device or self.k[0].device)
+
+    def slot_view(self, slot: int, length: int, n: int = 0) -> "KVCache":
+        """One slot as a batch-1 cache that already holds ``length`` tokens (chunked / suffix prefill)."""
+        view = KVCache.__new__(KVCache)
+        view.k = [t[slot:slot + 1] for t in self.k]
+        view.v = [t[slot:slot + 1] for t in self.v]
+        view.len, view.max_len, view.batch, view.pos = length, self.max_len, 1, None
+        view._rows = self._rows[:1]
+        return view
+
     def start_decode(self, lens: torch.Tensor):
         self.pos = lens.to(torch.long).clone()
+
+    def get_seq_length(self) -> int:
+        return self.len
+
+
+class SeqBatch:
+    """One engine step over a :class:`SeqStateCache`: the step's tokens packed back to back ``[1, T]`` plus, for each
+    sequence in it, its state slot and the position of its first token in this step.
+
+    A fresh prompt starts at 0 (its slot's old state is ignored), a continued prompt or a decode step starts where
+    the slot's sequence stands.  Kernels take :attr:`desc` — ``[seq_off (B+1), slots (B), pos0 (B), tok_seq (T),
+    tok_pos (T)]`` int32 on the device — and :attr:`live` (``[B]`` int32 or ``None``: rows whose state must not be
+    touched carry 0).  ``positions`` / ``last`` mirror :class:`PackedPrefill` for the engine."""
+
+    def __init__(self, cache: "SeqStateCache", desc, host, live=None, max_pos: int | None = None, T: int = 0):
+        self.cache, self.desc, self._host, self.live = cache, desc, host, live
+        self.B, self.T = int(desc[1].numel()), T
+        self.max_pos = cache.max_len if max_pos is None else max_pos      # bound on any key position this step
+        self.decode = host is None
+        self.positions = desc[4][None]
+        self.len, self.pos = 0, None                                      # KVCache duck-typing (unused)
+        self.cache_idx = desc[1].long()[desc[3].long()] * cache.max_len + desc[4].long()
+        self.last = (desc[0][1:] - 1).long()
+
+    @classmethod
+    def packed(cls, cache: "SeqStateCache", slots: list[int], lens: list[int], starts: list[int] | None = None):
+        starts = list(starts) if starts is not None else [0] * len(lens)
+        assert len(slots) == len(lens) == len(starts) and all(n > 0 for n in lens)
+        if any(s < 0 or s >= cache.batch for s in slots) or len(set(slots)) != len(slots):
+            raise ValueError(f"slots {slots}: each must be a distinct row of the cache (0..{cache.batch - 1})")
+        if any(p + n > cache.max_len for p, n in zip(starts, lens)):
+            raise ValueError(f"a sequence would pass the cache's {cache.max_len} positions")
+        off = [0]
+        for n in lens:
+            off.append(off[-1] + n)
+        tok_seq = torch.cat([torch.full((n,), b, dtype=torch.int32) for b, n in enumerate(lens)])
+        tok_pos = torch.cat([torch.arange(p, p + n, dtype=torch.int32) for p, n in zip(starts, lens)])
+        flat = torch.cat([torch.tensor(off + list(slots) + starts, dtype=torch.int32), tok_seq, tok_pos])
+        flat = flat.to(cache.device)
+        B, T = len(lens), off[-1]
+        desc = list(torch.split(flat, [B + 1, B, B, T, T]))
+        return cls(cache, desc, (off, list(slots), starts), None, max(p + n for p, n in zip(starts, lens)), T)
+
+    @classmethod
+    def decoding(cls, cache: "SeqStateCache", n: int):
+        """Rows ``[0, n)`` each advance by one token from ``cache.pos`` (a device tensor: no host sync, capturable)."""
+        ar = cache._arange[:n + 1]
+        pos = cache.pos[:n]
+        return cls(cache, [ar, ar[:n], pos, ar[:n], pos], None, cache.live[:n], None, n)
+
+    def host(self):
+        if self._host is None:      # decode rows on the CPU path: read the positions back
+            n = self.B
+            return list(range(n + 1)), list(range(n)), [int(p) for p in self.desc[2].tolist()]
+        return self._host
+
+    def is_live(self, b: int) -> bool:
+        return self.live is None or bool(self.live[b])
+
+
+class SeqStateCache:
+    """Per-slot sequence state for models whose layers are not all plain attention: every layer names the tensors
+    it keeps per sequence — K/V rows ``[slots, max_len, C]`` for attention, recurrent matrices and the carried inputs
+    of short convolutions ``[slots, ...]`` — and the cache allocates them for ``batch`` slots, like :class:`KVCache`
+    does for K/V alone.  ``pos`` (int32, device) is each slot's next position; a slot is recycled by starting its
+    next sequence at position 0, which makes every kernel ignore what the slot held.
+
+    ``specs``: per layer a dict ``name -> (shape after the slot axis, "act" | "f32" | "kv")``; ``"kv"`` entries get
+    the ``max_len`` axis, ``"act"`` ones the activation dtype."""
+
+    def __init__(self, specs: list[dict], batch: int, max_len: int, dtype, device):
+        self.specs, self.batch, self.max_len, self.dtype, self.device = specs, batch, max_len, dtype, torch.device(device)
+        self.layers: list[dict[str, torch.Tensor]] = []
+        for spec in specs:
+            d = {}
+            for name, (shape, kind) in spec.items():
+                full = (batch, max_len, *shape) if kind == "kv" else (batch, *shape)
+                d[name] = torch.zeros(full, dtype=torch.float32 if kind == "f32" else dtype, device=device)
+            self.layers.append(d)
+        self.pos = torch.zeros(batch, dtype=torch.int32, device=device)
+        self.live = torch.ones(batch, dtype=torch.int32, device=device)    # rows whose state a decode step may touch
+        self.len = 0
+        self.decoding = False             # generate(): set by start_decode, rows then advance one token per call
+        self.decode_splits = 1            # key splits of decode attention (fixed per cache: graph-capturable)
+        self._arange = torch.arange(batch + 1, dtype=torch.int32, device=device)
+
+    @staticmethod
+    def slot_bytes(specs: list[dict], max_len: int, dtype) -> int:
+        import math
+        el = torch.finfo(dtype).bits // 8
+        return sum(math.prod(shape) * (max_len * el if kind == "kv" else el if kind == "act" else 4)
+                   for spec in specs for shape, kind in spec.values())
+
+    # ---- the views the engine and generate() ask a cache for
+    def packed(self, slots: list[int], lens: list[int], device=None) -> SeqBatch:
+        return SeqBatch.packed(self, slots, lens)
+
+    def slot_view(self, slot: int, length: int, n: int) -> SeqBatch:
+        """``n`` more tokens of the sequence in ``slot`` that already holds ``length``."""
+        return SeqBatch.packed(self, [slot], [n], [length])
+
+    def head_rows(self, n: int) -> SeqBatch:
+        return SeqBatch.decoding(self, n)
+
+    def set_live(self, rows: list[int], n: int):
+        """Decode steps run rows ``[0, n)``; only ``rows`` may change their state (idle rows and rows in the middle
+        of a chunked prefill must not)."""
+        mask = torch.zeros(self.batch, dtype=torch.int32)
+        mask[rows] = 1
+        self.live.copy_(mask.to(self.device), non_blocking=True)
+
+    def start_decode(self, lens: torch.Tensor):
+        self.pos = lens.to(torch.int32).clone()
+        self.decoding = True
 
     def get_seq_length(self) -> int:
         return self.len

@@ -40,6 +40,34 @@ def native():
     return _C
 
 
+_SEQ = None
+
+
+def native_seq():
+    """The sequence-state kernels (``llm_in_practise_amd._seq``: recurrent mixers, short convolutions,
+    head-mixing attention, float-residual norms).  A small extension of its own: built in-tree on first use if
+    missing (three HIP files and the bindings), like the host extension."""
+    global _SEQ
+    if _SEQ is None:
+        try:
+            _SEQ = importlib.import_module("llm_in_practise_amd._seq")
+        except ImportError:
+            from ..csrc.build import build_seq_extension
+            build_seq_extension()
+            importlib.invalidate_caches()
+            _SEQ = importlib.import_module("llm_in_practise_amd._seq")
+    return _SEQ
+
+
+def use_seq(t: torch.Tensor) -> bool:
+    """True when a sequence-state op must run on the ``_seq`` HIP kernels (GPU tensors; raises if they cannot be
+    built or loaded — no eager fallback on a GPU box)."""
+    if t.is_cuda and not force_reference():
+        native_seq()
+        return True
+    return False
+
+
 def has_native() -> bool:
     try:
         native()

@@ -45,3 +45,14 @@ def gelu(x: torch.Tensor) -> torch.Tensor:
     if use_native(x) and x.is_contiguous():
         return fn_apply(_GeluFn, x)
     return F.gelu(x)
+
+
+def polynorm(z: torch.Tensor, coef: torch.Tensor, eps: float) -> torch.Tensor:
+    """PolyNorm activation over the last dimension: ``c0 N(z) + c1 N(z^2) + c2 N(z^3) + c3`` with ``N`` the division
+    by the root mean square (eps inside the root) and element-wise powers; ``coef`` float ``[4]``.  Statistics in
+    float; HIP kernel: one pass for the three sums, one to write (csrc/kernels/seq/seq_norms.hip)."""
+    from . import reference as ref
+    from ._native import native_seq, use_seq
+    if use_seq(z):
+        return native_seq().polynorm(z.contiguous(), coef, eps)
+    return ref.polynorm(z, coef, eps)

@@ -154,3 +154,17 @@ def sdpa_bshd(q, k, v, causal=True, scale=None, dropout_p=0.0, window=None, key_
             return o.view(B, S, Hq, D).to(dt)
     return ref.attention(q, k, v, causal=causal, scale=scale, dropout_p=dropout_p, window=window,
                          key_padding_mask=key_padding_mask)
+
+
+def talking_heads_attention(q, k_cache, v_cache, talk, gate_pre, heads: int, kv_heads: int, scale: float, sb,
+                            nsplit: int = 1):
+    """Causal softmax attention over a slot-indexed cache whose softmax WEIGHTS are mixed across heads before they
+    meet the values: ``w'_h = sum_g talk[h, g] w_g``; head ``h`` applies ``w'_h`` to the values of its own kv head.
+    ``q`` ``[T, H*dk]`` for the step's packed tokens; ``k_cache`` / ``v_cache`` ``[slots, max_len, G*dk | G*dv]``
+    already hold the step's keys and values at their positions; ``gate_pre`` ``[T, H*dv]`` is the pre-activation of
+    the sigmoid output gate.  Returns ``[T, H*dv]``.  Scores, weights and the mixing are float.  ``nsplit`` cuts the
+    keys of each query into that many independent sweeps (decode over long caches)."""
+    from ._native import native_seq, use_seq
+    if use_seq(q):
+        return native_seq().talk_attention(q, k_cache, v_cache, talk, gate_pre, heads, kv_heads, scale, nsplit, sb.desc)
+    return ref.talk_attention(q, k_cache, v_cache, talk, gate_pre, heads, kv_heads, scale, sb)

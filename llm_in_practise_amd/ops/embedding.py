@@ -102,3 +102,21 @@ class Embedding(nn.Embedding):
         if self.max_norm is not None or self.sparse or self.scale_grad_by_freq:
             return super().forward(ids)
         return embedding(ids, self.weight, self.padding_idx)
+
+
+def sinusoid_inv_freq(width: int, base: float = 10000.0) -> torch.Tensor:
+    """``base^(-2i / width)`` for i < ceil(width / 2), evaluated in float64 and rounded once to float."""
+    i = torch.arange((width + 1) // 2, dtype=torch.float64)
+    return (base ** (-2.0 * i / width)).float()
+
+
+def embed_sincos(tokens: torch.Tensor, positions: torch.Tensor, table: torch.Tensor, inv_freq: torch.Tensor,
+                 scale: float) -> torch.Tensor:
+    """Scaled token embedding plus the interleaved sinusoidal position vector (even entries sin, odd entries cos of
+    ``position * inv_freq[i]``), as a float ``[T, width]`` residual stream; angles in float."""
+    from . import reference as ref
+    from ._native import native_seq, use_seq
+    if use_seq(table):
+        return native_seq().embed_sincos(tokens.reshape(-1).long().contiguous(),
+                                         positions.reshape(-1).int().contiguous(), table, inv_freq, scale)
+    return ref.embed_sincos(tokens, positions, table, inv_freq, scale)

@@ -111,3 +111,43 @@ class LayerNorm(nn.LayerNorm):
 
     def forward(self, x):
         return layer_norm(x, self.weight, self.bias, self.eps)
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# Float residual stream (inference): models that keep the residual sum in 32 bits while their matrix products run
+# in bf16.  HIP kernels: csrc/kernels/seq/seq_norms.hip.
+def rms_norm_f32(x: torch.Tensor, weight: torch.Tensor, eps: float, dtype: torch.dtype) -> torch.Tensor:
+    """RMS norm of a float tensor, written in the activation ``dtype`` (bf16 or float)."""
+    from ._native import native_seq, use_seq
+    if use_seq(x):
+        return native_seq().rms_f32(x, weight, eps, dtype == torch.bfloat16)
+    return ref.rms_f32(x, weight, eps, dtype)
+
+
+def gated_residual_norm(x: torch.Tensor, y: torch.Tensor, gate_pre: torch.Tensor, gate_bias: torch.Tensor,
+                        post_weight: torch.Tensor, next_weight: torch.Tensor | None, eps: float):
+    """The sublayer exit of a gated, post-normed residual block, in place on the float residual ``x``:
+    ``x += rmsnorm(y * sigmoid(gate_pre + gate_bias)) * post_weight``; with ``next_weight`` also returns
+    ``rmsnorm(x) * next_weight`` (the next sublayer's input) from the same kernel."""
+    from ._native import native_seq, use_seq
+    if use_seq(x):
+        return native_seq().gated_residual(x, y, gate_pre, gate_bias, post_weight, next_weight, eps)
+    return ref.gated_residual(x, y, gate_pre, gate_bias, post_weight, next_weight, eps)
+
+
+def dual_norm_mean(a: torch.Tensor, b: torch.Tensor, wa: torch.Tensor, wb: torch.Tensor, eps: float) -> torch.Tensor:
+    """``0.5 * (rmsnorm(a) * wa + rmsnorm(b) * wb)``: two branches of a layer joined at equal weight."""
+    from ._native import native_seq, use_seq
+    if use_seq(a):
+        return native_seq().dual_norm_mean(a, b, wa, wb, eps)
+    return ref.dual_norm_mean(a, b, wa, wb, eps)
+
+
+def head_norm_gate(o: torch.Tensor, weight: torch.Tensor, gate_pre: torch.Tensor, eps: float) -> torch.Tensor:
+    """Read-out of a recurrent mixer: ``o`` float ``[T, H, dv]`` is RMS-normed per head, scaled by ``weight``
+    (``[dv]`` shared by the heads or ``[H * dv]``) and multiplied by ``sigmoid(gate_pre)``; returns ``[T, H * dv]``
+    in ``gate_pre``'s dtype."""
+    from ._native import native_seq, use_seq
+    if use_seq(o):
+        return native_seq().head_norm_gate(o, weight, gate_pre, eps)
+    return ref.head_norm_gate(o, weight, gate_pre, eps)

@@ -1,0 +1,43 @@
+"""Matrix-memory recurrences over packed variable-length batches with per-slot float state.
+
+* :func:`mlstm_scan` — the mLSTM cell of xLSTM with exponential gating stabilised by a running maximum.
+* :func:`gated_delta_scan` — the delta rule with a per-key-channel decay (erase, then write the prediction error).
+
+Both keep ``S`` as ``[slots, H, dv, dk]`` float (one column of the ``[dk, dv]`` matrix contiguous), read
+and write it in place, and treat a sequence that starts at position 0 as starting from zero state.  The same kernel
+serves prefill (a scan over the step's tokens with the state in registers) and decode (one token: load, update,
+store).  HIP kernels: csrc/kernels/seq/seq_scan.hip; the CPU path is ops/reference.py.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import reference as ref
+from ._native import native_seq, use_seq
+
+
+def mlstm_scan(q, k, v, i_pre, f_pre, i_bias, f_bias, cap: float, q_scale: float, S, N, M, heads: int, sb):
+    """``q, k`` ``[T, H*dk]``, ``v`` ``[T, H*dv]`` (activation dtype), gate pre-activations float ``[T, H]``.
+    Gates: ``i = cap*tanh((i_pre+i_bias)/cap)``, ``f = logsigmoid(cap*tanh((f_pre+f_bias)/cap))``; running maximum
+    ``m`` starts at 0.  Returns float ``[T, H, dv]``: ``S^T q / (max(|n.q|, exp(-m)) + 1e-6)``."""
+    if use_seq(q):
+        return native_seq().mlstm_scan(q, k, v, i_pre, f_pre, i_bias, f_bias, cap, q_scale, S, N, M, heads, sb.desc,
+                                       sb.live)
+    return ref.mlstm_scan(q, k, v, i_pre, f_pre, i_bias, f_bias, cap, q_scale, S, N, M, heads, sb)
+
+
+def decay_gate(pre, bias, a_log, dk: int):
+    """``exp(-exp(a_log[h]) * softplus(pre + bias))`` laid out ``[T, H*dk]``, float."""
+    if use_seq(pre):
+        return native_seq().decay_gate(pre.contiguous(), bias, a_log, dk)
+    return ref.decay_gate(pre, bias, a_log, dk)
+
+
+def gated_delta_scan(q, k, v, g, beta_pre, S, heads: int, kv_heads: int, sb):
+    """``q, k`` ``[T, G*dk]`` (already unit vectors, q scaled), ``v`` ``[T, H*dv]``, ``g`` float ``[T, H*dk]`` decays,
+    ``beta_pre`` float ``[T, H]``.  Per head: ``S <- g*S; u = sigmoid(beta_pre)*(v - S^T k); S <- S + k u^T;
+    o = S^T q``.  Returns float ``[T, H, dv]``."""
+    if use_seq(q):
+        return native_seq().delta_scan(q, k, v, g.contiguous(), beta_pre.contiguous(), S, heads, kv_heads, sb.desc,
+                                       sb.live)
+    return ref.delta_scan(q, k, v, g, beta_pre, S, heads, kv_heads, sb)

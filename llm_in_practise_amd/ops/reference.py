@@ -144,3 +144,149 @@ def adamw_step(p, g, m, v, step: int, lr: float, beta1: float, beta2: float, eps
     bc2 = 1 - beta2 ** step
     denom = (v / bc2).sqrt().add_(eps)
     p.addcdiv_(m, denom, value=-lr / bc1)
+
+
+# ----------------------------------------------------------------------------- sequence-state ops
+# Packed variable-length batches with per-slot state (models/common.py ``SeqBatch``): ``sb.host()`` gives
+# (offsets, slots, first positions) as lists.  States are float and updated in place; a sequence whose first
+# position is 0 starts from zero state whatever its slot held.
+def embed_sincos(tok, pos, table, inv_freq, scale: float):
+    x = table[tok.reshape(-1)].float() * scale
+    ang = pos.reshape(-1).float()[:, None] * inv_freq[None, :].float()
+    w = x.shape[1]
+    x[:, 0::2] += torch.sin(ang)[:, :(w + 1) // 2]
+    x[:, 1::2] += torch.cos(ang)[:, :w // 2]
+    return x
+
+
+def _unit_rms(x, eps):
+    return x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps)
+
+
+def rms_f32(x, w, eps: float, dtype):
+    return (_unit_rms(x.float(), eps) * w).to(dtype)
+
+
+def gated_residual(x, y, r, b, wb, wn, eps: float):
+    z = y.float() * torch.sigmoid(r.float() + b)
+    x += _unit_rms(z, eps) * wb
+    return None if wn is None else (_unit_rms(x, eps) * wn).to(y.dtype)
+
+
+def dual_norm_mean(a, b, wa, wb, eps: float):
+    return (0.5 * (_unit_rms(a.float(), eps) * wa + _unit_rms(b.float(), eps) * wb)).to(a.dtype)
+
+
+def polynorm(z, coef, eps: float):
+    zf = z.float()
+    out = coef[3] + sum(coef[i] * _unit_rms(zf ** (i + 1), eps) for i in range(3))
+    return out.to(z.dtype)
+
+
+def head_norm_gate(o, w, gate, eps: float):
+    T, H, dv = o.shape
+    y = _unit_rms(o, eps) * (w.view(H, dv) if w.numel() != dv else w)
+    return (y.reshape(T, H * dv) * torch.sigmoid(gate.float())).to(gate.dtype)
+
+
+def decay_gate(pre, bias, a_log, dk: int):
+    T, HD = pre.shape
+    dt = F.softplus(pre + bias).view(T, HD // dk, dk)
+    return torch.exp(-torch.exp(a_log)[None, :, None] * dt).reshape(T, HD)
+
+
+def short_conv(u, w, state, segs, seg_w, seg_scale, sb, eps: float, out_f32: bool):
+    T, C = u.shape
+    taps = w.shape[1]
+    off, slots, pos0 = sb.host()
+    y = torch.empty(T, C, dtype=torch.float32, device=u.device)
+    for b, slot in enumerate(slots):
+        a, e = off[b], off[b + 1]
+        if taps > 1:
+            prev = state[slot].float() if pos0[b] > 0 else torch.zeros(taps - 1, C, device=u.device)
+            ext = torch.cat([prev, u[a:e].float()], 0)
+            if sb.is_live(b):
+                state[slot] = ext[-(taps - 1):].to(state.dtype)
+        else:
+            ext = u[a:e].float()
+        win = ext.unfold(0, taps, 1)                       # [len, C, taps]
+        y[a:e] = (win * w[None]).sum(-1)
+    out = torch.empty_like(y)
+    for (c0, nh, hw, mode), sw, sc in zip(segs, seg_w, seg_scale):
+        v = y[:, c0:c0 + nh * hw].view(T, nh, hw)
+        if mode >= 2:
+            v = F.silu(v)
+        if mode == 1:
+            v = _unit_rms(v, eps) * sw
+        elif mode == 3:
+            v = v * torch.rsqrt(v.pow(2).sum(-1, keepdim=True) + 1e-6) * sc
+        out[:, c0:c0 + nh * hw] = v.reshape(T, nh * hw)
+    return out if out_f32 else out.to(u.dtype)
+
+
+def mlstm_scan(q, k, v, ipre, fpre, ib, fb, cap: float, qscale: float, S, N, M, H: int, sb):
+    T = q.shape[0]
+    dk, dv = q.shape[1] // H, v.shape[1] // H
+    qf, kf, vf = q.float().view(T, H, dk) * qscale, k.float().view(T, H, dk), v.float().view(T, H, dv)
+    ig = cap * torch.tanh((ipre + ib) / cap)
+    fg = F.logsigmoid(cap * torch.tanh((fpre + fb) / cap))
+    out = torch.empty(T, H, dv, dtype=torch.float32, device=q.device)
+    off, slots, pos0 = sb.host()
+    for b, slot in enumerate(slots):
+        if not sb.is_live(b):
+            continue
+        fresh = pos0[b] == 0
+        s = torch.zeros_like(S[slot]) if fresh else S[slot].clone()         # [H, dv, dk]
+        n = torch.zeros_like(N[slot]) if fresh else N[slot].clone()         # [H, dk]
+        m = torch.zeros_like(M[slot]) if fresh else M[slot].clone()         # [H]
+        for t in range(off[b], off[b + 1]):
+            mn = torch.maximum(fg[t] + m, ig[t])
+            a, c = torch.exp(fg[t] + m - mn), torch.exp(ig[t] - mn)
+            m = mn
+            s = a[:, None, None] * s + c[:, None, None] * vf[t][:, :, None] * kf[t][:, None, :]
+            n = a[:, None] * n + c[:, None] * kf[t]
+            den = torch.maximum((n * qf[t]).sum(-1).abs(), torch.exp(-m)) + 1e-6
+            out[t] = (s * qf[t][:, None, :]).sum(-1) / den[:, None]
+        S[slot], N[slot], M[slot] = s, n, m
+    return out
+
+
+def delta_scan(q, k, v, g, bpre, S, H: int, G: int, sb):
+    T = q.shape[0]
+    dk, dv = q.shape[1] // G, v.shape[1] // H
+    rep = H // G
+    qf = q.float().view(T, G, dk).repeat_interleave(rep, 1)
+    kf = k.float().view(T, G, dk).repeat_interleave(rep, 1)
+    vf, gf, beta = v.float().view(T, H, dv), g.view(T, H, dk), torch.sigmoid(bpre)
+    out = torch.empty(T, H, dv, dtype=torch.float32, device=q.device)
+    off, slots, pos0 = sb.host()
+    for b, slot in enumerate(slots):
+        if not sb.is_live(b):
+            continue
+        s = torch.zeros_like(S[slot]) if pos0[b] == 0 else S[slot].clone()   # [H, dv, dk]
+        for t in range(off[b], off[b + 1]):
+            s = s * gf[t][:, None, :]
+            u = beta[t][:, None] * (vf[t] - (s * kf[t][:, None, :]).sum(-1))
+            s = s + u[:, :, None] * kf[t][:, None, :]
+            out[t] = (s * qf[t][:, None, :]).sum(-1)
+        S[slot] = s
+    return out
+
+
+def talk_attention(q, kc, vc, talk, gate, H: int, G: int, scale: float, sb):
+    T = q.shape[0]
+    dk, dv = q.shape[1] // H, vc.shape[2] // G
+    rep = H // G
+    out = torch.empty(T, H * dv, dtype=torch.float32, device=q.device)
+    off, slots, pos0 = sb.host()
+    for b, slot in enumerate(slots):
+        a, e = off[b], off[b + 1]
+        L = pos0[b] + e - a
+        kk = kc[slot, :L].float().view(L, G, dk).repeat_interleave(rep, 1)      # [L, H, dk]
+        vv = vc[slot, :L].float().view(L, G, dv).repeat_interleave(rep, 1)
+        sc = torch.einsum("thd,lhd->htl", q[a:e].float().view(e - a, H, dk), kk) * scale
+        vis = torch.arange(L, device=q.device)[None, :] <= (pos0[b] + torch.arange(e - a, device=q.device))[:, None]
+        w = torch.softmax(sc.masked_fill(~vis[None], float("-inf")), -1)
+        w = torch.einsum("hg,gtl->htl", talk, w)
+        out[a:e] = torch.einsum("htl,lhd->thd", w, vv).reshape(e - a, H * dv)
+    return (out * torch.sigmoid(gate.float())).to(q.dtype)
