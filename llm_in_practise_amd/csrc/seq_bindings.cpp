@@ -7,6 +7,7 @@
 
 #include <vector>
 
+namespace lipa {
 struct SeqDesc {
   const int* seq_off;
   const int* slots;
@@ -16,6 +17,8 @@ struct SeqDesc {
   const int* live;
   int B, Ttot;
 };
+}  // namespace lipa
+using lipa::SeqDesc;
 
 void seq_embed_sincos(int, const long*, const int*, const void*, const float*, float*, int, int, float, hipStream_t);
 void seq_rms_f32(int, const float*, const float*, void*, int, int, float, hipStream_t);
