@@ -1,7 +1,7 @@
 """Plain, slow Mobupel: one function per mechanism, token by token, float64 on the CPU.
 
 This is the yardstick of the Mobupel tests.  It shares nothing with the product path
-(``llm_in_practise_amd/models/mobupel.py``, ``ops/recurrent.py``, ``ops/seqmix.py`` and the HIP
+(``llm_in_practise_amd/models/mobupel.py``, ``ops/recurrent.py``, ``ops/conv.py``, ``ops/reference.py`` and the HIP
 kernels): no packed batches, no slots, no cache object — every function takes one sequence,
 ``[tokens, features]``, and loops over its tokens where the mechanism is recurrent.
 
@@ -23,10 +23,6 @@ def rms_unit(x, eps):
 
 def rms_norm(x, w, eps):
     return rms_unit(x, eps) * w
-
-
-def gelu_tanh(z):
-    return 0.5 * z * (1 + torch.tanh(math.sqrt(2 / math.pi) * (z + 0.044715 * z ** 3)))
 
 
 def embed(tokens, table, scale, width, start=0):
@@ -172,10 +168,10 @@ def forward(cfg, weights, tokens, return_layers=False):
 
 
 def random_weights(cfg, seed=0, dtype=torch.float32):
-    """Random tensors of the shapes a config asks for (ranks of the low-rank gates: ``rank``)."""
+    """Random tensors of the shapes a config asks for (inner sizes of the two low-rank gates: ``_rank_a``, ``_rank_g``)."""
     g = torch.Generator().manual_seed(seed)
     Wd, V = cfg["width"], cfg["vocab"]
-    rank = cfg.get("_rank", 8)
+    rank_a, rank_g = cfg.get("_rank_a", 8), cfg.get("_rank_g", 5)
 
     def lin(o, i, s=1.0):
         return (torch.randn(o, i, generator=g) * s / math.sqrt(i)).to(dtype)
@@ -199,10 +195,11 @@ def random_weights(cfg, seed=0, dtype=torch.float32):
         else:
             l, r = m["left"], m["right"]
             q = p + "mix.left."
-            H, G, dk, dv, taps = l["heads"], l["kv_heads"], l["dim"], l["vdim"], l["conv"]
+            H, G, dk, dv, taps = l["heads"], l["kv_heads"], l["dim"], l["vdim"], l.get("conv", 0)
             W[q + "q"], W[q + "k"], W[q + "v"] = lin(H * dk, Wd), lin(G * dk, Wd), lin(G * dv, Wd)
             for n, c in (("q", H * dk), ("k", G * dk), ("v", G * dv)):
-                W[q + n + ".conv"] = (torch.randn(c, taps, generator=g) * 0.5).to(dtype)
+                if taps:
+                    W[q + n + ".conv"] = (torch.randn(c, taps, generator=g) * 0.5).to(dtype)
             W[q + "q.norm"], W[q + "k.norm"] = vec(dk), vec(dk)
             W[q + "talk"] = (torch.eye(H) + 0.3 * torch.randn(H, H, generator=g)).to(dtype)
             W[q + "g"], W[q + "o"] = lin(H * dv, Wd), lin(Wd, H * dv)
@@ -213,8 +210,8 @@ def random_weights(cfg, seed=0, dtype=torch.float32):
                 W[q + n + ".conv"] = (torch.randn(c, taps, generator=g) * 0.5).to(dtype)
             W[q + "b"], W[q + "A_log"] = lin(H, Wd), vec(H, -3.0, 0.0)
             W[q + "norm"] = vec(dv)
-            W[q + "a1"], W[q + "a2"], W[q + "dt_bias"] = lin(rank, Wd), lin(H * dk, rank), vec(H * dk, -3.0, 0.0)
-            W[q + "g1"], W[q + "g2"], W[q + "o"] = lin(rank, Wd), lin(H * dv, rank), lin(Wd, H * dv)
+            W[q + "a1"], W[q + "a2"], W[q + "dt_bias"] = lin(rank_a, Wd), lin(H * dk, rank_a), vec(H * dk, -3.0, 0.0)
+            W[q + "g1"], W[q + "g2"], W[q + "o"] = lin(rank_g, Wd), lin(H * dv, rank_g), lin(Wd, H * dv)
             W[p + "mix.left.out"], W[p + "mix.right.out"] = vec(Wd), vec(Wd)
         if lc.get("mlp") is not None:
             ff = lc["mlp"]["ff"]
