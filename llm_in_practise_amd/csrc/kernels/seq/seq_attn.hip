@@ -73,6 +73,118 @@ __global__ __launch_bounds__(64) void k_talk_attn_partial(const T* __restrict__ 
   }
 }
 
+
+// ------------------------------------------------------------------------------------------------ MFMA pass 1 (bf16)
+// One wave per (tile of up to 32 consecutive queries of one sequence, query head g, kv head c of the VALUES, key
+// split).  Scores are computed transposed, S^T[key][query] = K Q^T with v_mfma_f32_32x32x16_bf16: a lane then owns one
+// query (lane % 32) and 16 of the tile's 32 keys, so the softmax statistics are lane-local plus one exchange between
+// the wave's halves, and the weights P^T are already laid out as the B operand of O^T[col][query] += V^T P^T.  The
+// value tile goes through LDS row-major (16 B stores); a lane picks its column's 8 keys of a step with 2-byte reads.
+// K and Q operands are 16 B global loads (Q stays in registers).  Rows past the cache end are clamped: their weights
+// are 0.  Writes the same partial format as the scalar kernel: m, l per (token, g, split) and unnormalised U columns
+// [c*dv, (c+1)*dv).
+template <int NDS, int NDT>
+__global__ __launch_bounds__(64) void k_talk_attn_mfma(const bf16* __restrict__ q, int ldq, const bf16* __restrict__ kc,
+                                                       const bf16* __restrict__ vc, float* __restrict__ pm,
+                                                       float* __restrict__ pl, float* __restrict__ pu,
+                                                       const int* __restrict__ tile_seq, const int* __restrict__ tile_t0,
+                                                       int H, int G, int dk, int dv, int max_len, int nsplit,
+                                                       float scale, SeqDesc d) {
+  constexpr int LDMAX = NDT * 32 + 8;
+  __shared__ __attribute__((aligned(16))) bf16 sV[32 * LDMAX];
+  const int tile = blockIdx.x, g = blockIdx.y, c = blockIdx.z % G, z = blockIdx.z / G;
+  const int lane = threadIdx.x, hi = lane >> 5, ql = lane & 31;
+  const int s = tile_seq[tile], t0 = tile_t0[tile], tend = d.seq_off[s + 1], slot = d.slots[s];
+  const int tq = min(t0 + ql, tend - 1);
+  const bool valid_q = t0 + ql < tend;
+  const int pos_q = d.tok_pos[tq], pmax = d.tok_pos[min(t0 + 31, tend - 1)];
+  const int nds = dk >> 4, ndt = dv >> 5, LD = dv + 8, GV = G * dv, kh = g / (H / G);
+  const int per = (pmax + nsplit) / nsplit, j0 = z * per, j1 = min(pmax + 1, j0 + per);
+  const bf16* kbase = kc + ((size_t)slot * max_len) * (G * dk) + kh * dk + 8 * hi;
+  const bf16* vbase = vc + ((size_t)slot * max_len) * GV + c * dv;
+  bf16x8 qf[NDS];
+#pragma unroll
+  for (int ds = 0; ds < NDS; ++ds)
+    if (ds < nds) qf[ds] = *reinterpret_cast<const bf16x8*>(q + (size_t)tq * ldq + g * dk + 16 * ds + 8 * hi);
+  f32x16 acc[NDT];
+#pragma unroll
+  for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[dt][r] = 0.f;
+  float m = -INFINITY, l = 0.f;
+  const int vpr = dv >> 3;                       // 16 B vectors per value row
+  for (int jb = j0; jb < j1; jb += 32) {
+    __syncthreads();
+    for (int e = lane; e < 32 * vpr; e += 64) {
+      const int row = e / vpr, cv = e % vpr;
+      *reinterpret_cast<bf16x8*>(sV + row * LD + cv * 8) =
+          *reinterpret_cast<const bf16x8*>(vbase + (size_t)min(jb + row, max_len - 1) * GV + cv * 8);
+    }
+    f32x16 sc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) sc[r] = 0.f;
+    const bf16* kr = kbase + (size_t)min(jb + ql, max_len - 1) * (G * dk);
+#pragma unroll
+    for (int ds = 0; ds < NDS; ++ds)
+      if (ds < nds)
+        sc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<const bf16x8*>(kr + 16 * ds), qf[ds], sc, 0, 0, 0);
+    float mt = -INFINITY;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int key = jb + (r & 3) + 8 * (r >> 2) + 4 * hi;
+      sc[r] = (key <= pos_q && key < j1) ? sc[r] * scale : -INFINITY;
+      mt = fmaxf(mt, sc[r]);
+    }
+    mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+    const float mn = fmaxf(m, mt), ms = mn == -INFINITY ? 0.f : mn;
+    const float corr = expf(m - ms);
+    float rs = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      sc[r] = expf(sc[r] - ms);
+      rs += sc[r];
+    }
+    rs += __shfl_xor(rs, 32, 64);
+    l = l * corr + rs;
+    m = mn;
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[dt][r] *= corr;
+    __syncthreads();
+#pragma unroll
+    for (int u2 = 0; u2 < 2; ++u2) {
+      bf16x8 pb;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) pb[j] = (bf16)sc[8 * u2 + j];
+#pragma unroll
+      for (int dt = 0; dt < NDT; ++dt)
+        if (dt < ndt) {
+          bf16x8 vf;
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            const int r = 8 * u2 + j;
+            vf[j] = sV[((r & 3) + 8 * (r >> 2) + 4 * hi) * LD + dt * 32 + ql];
+          }
+          acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pb, acc[dt], 0, 0, 0);
+        }
+    }
+  }
+  if (!valid_q) return;
+  const size_t o = ((size_t)tq * H + g) * nsplit + z;
+  if (c == 0 && hi == 0) {
+    pm[o] = m;
+    pl[o] = l;
+  }
+#pragma unroll
+  for (int dt = 0; dt < NDT; ++dt)
+    if (dt < ndt)
+#pragma unroll
+      for (int r4 = 0; r4 < 4; ++r4)
+        *reinterpret_cast<f32x4*>(pu + o * GV + c * dv + dt * 32 + 8 * r4 + 4 * hi) =
+            f32x4{acc[dt][4 * r4], acc[dt][4 * r4 + 1], acc[dt][4 * r4 + 2], acc[dt][4 * r4 + 3]};
+}
+
 // out[t, h, c] = sigmoid(gate[t, h*dv + c]) * sum_g talk[h, g] * U_g[kv(h)*dv + c] / l_g   (splits merged first)
 template <typename T>
 __global__ __launch_bounds__(64) void k_talk_attn_merge(const float* __restrict__ pm, const float* __restrict__ pl,
@@ -101,10 +213,29 @@ __global__ __launch_bounds__(64) void k_talk_attn_merge(const float* __restrict_
 
 int seq_attn_max_cols() { return 64 * MAXC; }
 
+// the MFMA sweep needs bf16, 16-byte rows and whole operand tiles
+bool seq_attn_mfma_ok(int code, int ldq, int dk, int dv) {
+  return code == 0 && dk % 16 == 0 && dk <= 256 && dv % 32 == 0 && dv <= 256 && ldq % 8 == 0;
+}
+
 void seq_talk_attention(int code, const void* q, int ldq, const void* kc, const void* vc, float* pm, float* pl,
                         float* pu, const float* talk, const void* gate, int ldg, void* out, int H, int G, int dk, int dv,
-                        int max_len, int nsplit, float scale, SeqDesc d, hipStream_t st) {
+                        int max_len, int nsplit, float scale, const int* tile_seq, const int* tile_t0, int ntiles,
+                        SeqDesc d, hipStream_t st) {
   if (d.Ttot == 0) return;
+  if (tile_seq != nullptr && seq_attn_mfma_ok(code, ldq, dk, dv)) {
+    const dim3 grid(ntiles, H, G * nsplit);
+    if (dk <= 128 && dv <= 128)
+      hipLaunchKernelGGL((k_talk_attn_mfma<8, 4>), grid, dim3(64), 0, st, (const bf16*)q, ldq, (const bf16*)kc,
+                         (const bf16*)vc, pm, pl, pu, tile_seq, tile_t0, H, G, dk, dv, max_len, nsplit, scale, d);
+    else
+      hipLaunchKernelGGL((k_talk_attn_mfma<16, 8>), grid, dim3(64), 0, st, (const bf16*)q, ldq, (const bf16*)kc,
+                         (const bf16*)vc, pm, pl, pu, tile_seq, tile_t0, H, G, dk, dv, max_len, nsplit, scale, d);
+    hipLaunchKernelGGL(k_talk_attn_merge<bf16>, dim3(d.Ttot, H), dim3(64), 0, st, pm, pl, pu, talk, (const bf16*)gate,
+                       ldg, (bf16*)out, H, G, dv, nsplit);
+    LIPA_CHECK_LAUNCH();
+    return;
+  }
   SEQ_DISPATCH_T(code, {
     hipLaunchKernelGGL(k_talk_attn_partial<T>, dim3(d.Ttot, H, nsplit), dim3(64), sizeof(float) * dk, st, (const T*)q,
                        ldq, (const T*)kc, (const T*)vc, pm, pl, pu, H, G, dk, dv, max_len, nsplit, scale, d);

@@ -36,7 +36,8 @@ void seq_mlstm_scan(int, const void*, int, const void*, int, const void*, int, c
 void seq_delta_scan(int, const void*, int, const void*, int, const void*, int, const float*, const float*, float*,
                     float*, int, int, int, int, SeqDesc, hipStream_t);
 void seq_talk_attention(int, const void*, int, const void*, const void*, float*, float*, float*, const float*,
-                        const void*, int, void*, int, int, int, int, int, int, float, SeqDesc, hipStream_t);
+                        const void*, int, void*, int, int, int, int, int, int, float, const int*, const int*, int,
+                        SeqDesc, hipStream_t);
 int seq_scan_max_dk();
 int seq_conv_max_head();
 int seq_conv_max_taps();
@@ -280,8 +281,9 @@ Tensor delta_scan(Tensor q, Tensor k, Tensor v, Tensor g, Tensor bpre, Tensor S,
 }
 
 // q [T, H*dk]; kc [slots, max_len, G*dk], vc [slots, max_len, G*dv] already hold this step's keys and values
+// tiles (optional): [tile_seq, tile_t0] int32 — runs of up to 32 consecutive tokens of one sequence that cover the step
 Tensor talk_attention(Tensor q, Tensor kc, Tensor vc, Tensor talk, Tensor gate, int64_t H, int64_t G, double scale,
-                      int64_t nsplit, std::vector<Tensor> desc) {
+                      int64_t nsplit, std::vector<Tensor> desc, std::vector<Tensor> tiles) {
   const int code = code_of(q);
   const int64_t T = q.size(0);
   TORCH_CHECK(G >= 1 && H % G == 0 && q.dim() == 2 && q.size(1) % H == 0, "q: [T, H * dk]");
@@ -299,14 +301,25 @@ Tensor talk_attention(Tensor q, Tensor kc, Tensor vc, Tensor talk, Tensor gate, 
   TORCH_CHECK(talk.numel() == H * H, "talk: [H, H]");
   rows(gate, T, H * dv, code, "gate");
   SeqDesc d = desc_of(desc, optional<Tensor>(), T);
+  const int* tseq = nullptr;
+  const int* tt0 = nullptr;
+  int ntiles = 0;
+  if (tiles.size() == 2) {
+    for (auto& t : tiles) TORCH_CHECK(t.is_cuda() && t.scalar_type() == at::kInt && t.is_contiguous(), "tiles: int32");
+    TORCH_CHECK(tiles[0].numel() == tiles[1].numel(), "tiles: two arrays of one length");
+    tseq = tiles[0].data_ptr<int>();
+    tt0 = tiles[1].data_ptr<int>();
+    ntiles = (int)tiles[0].numel();
+    TORCH_CHECK((int64_t)ntiles * 32 >= T && G * nsplit <= 65535, "tiles must cover the tokens");
+  }
   auto fo = q.options().dtype(at::kFloat);
   auto pm = at::empty({T, H, nsplit}, fo), pl = at::empty({T, H, nsplit}, fo);
   auto pu = at::empty({T, H, nsplit, G * dv}, fo);
   auto out = at::empty({T, H * dv}, q.options());
   seq_talk_attention(code, q.data_ptr(), ld(q), kc.data_ptr(), vc.data_ptr(), pm.data_ptr<float>(),
                      pl.data_ptr<float>(), pu.data_ptr<float>(), talk.data_ptr<float>(), gate.data_ptr(), ld(gate),
-                     out.data_ptr(), (int)H, (int)G, (int)dk, (int)dv, (int)max_len, (int)nsplit, (float)scale, d,
-                     stream());
+                     out.data_ptr(), (int)H, (int)G, (int)dk, (int)dv, (int)max_len, (int)nsplit, (float)scale, tseq, tt0,
+                     ntiles, d, stream());
   return out;
 }
 

@@ -288,8 +288,10 @@ class SeqBatch:
     tok_pos (T)]`` int32 on the device — and :attr:`live` (``[B]`` int32 or ``None``: rows whose state must not be
     touched carry 0).  ``positions`` / ``last`` mirror :class:`PackedPrefill` for the engine."""
 
-    def __init__(self, cache: "SeqStateCache", desc, host, live=None, max_pos: int | None = None, T: int = 0):
+    def __init__(self, cache: "SeqStateCache", desc, host, live=None, max_pos: int | None = None, T: int = 0,
+                 tiles=None):
         self.cache, self.desc, self._host, self.live = cache, desc, host, live
+        self.tiles = tiles or []          # [tile_seq, tile_t0]: runs of <= 32 tokens of one sequence (attention tiles)
         self.B, self.T = int(desc[1].numel()), T
         self.max_pos = cache.max_len if max_pos is None else max_pos      # bound on any key position this step
         self.decode = host is None
@@ -311,18 +313,21 @@ class SeqBatch:
             off.append(off[-1] + n)
         tok_seq = torch.cat([torch.full((n,), b, dtype=torch.int32) for b, n in enumerate(lens)])
         tok_pos = torch.cat([torch.arange(p, p + n, dtype=torch.int32) for p, n in zip(starts, lens)])
-        flat = torch.cat([torch.tensor(off + list(slots) + starts, dtype=torch.int32), tok_seq, tok_pos])
+        tile_seq = [b for b, n in enumerate(lens) for _ in range(0, n, 32)]
+        tile_t0 = [off[b] + i for b, n in enumerate(lens) for i in range(0, n, 32)]
+        flat = torch.cat([torch.tensor(off + list(slots) + starts + tile_seq + tile_t0, dtype=torch.int32), tok_seq, tok_pos])
         flat = flat.to(cache.device)
-        B, T = len(lens), off[-1]
-        desc = list(torch.split(flat, [B + 1, B, B, T, T]))
-        return cls(cache, desc, (off, list(slots), starts), None, max(p + n for p, n in zip(starts, lens)), T)
+        B, T, nt = len(lens), off[-1], len(tile_seq)
+        parts = list(torch.split(flat, [B + 1, B, B, nt, nt, T, T]))
+        desc = parts[:3] + parts[5:]
+        return cls(cache, desc, (off, list(slots), starts), None, max(p + n for p, n in zip(starts, lens)), T, parts[3:5])
 
     @classmethod
     def decoding(cls, cache: "SeqStateCache", n: int):
         """Rows ``[0, n)`` each advance by one token from ``cache.pos`` (a device tensor: no host sync, capturable)."""
         ar = cache._arange[:n + 1]
         pos = cache.pos[:n]
-        return cls(cache, [ar, ar[:n], pos, ar[:n], pos], None, cache.live[:n], None, n)
+        return cls(cache, [ar, ar[:n], pos, ar[:n], pos], None, cache.live[:n], None, n, [ar[:n], ar[:n]])
 
     def host(self):
         if self._host is None:      # decode rows on the CPU path: read the positions back

@@ -166,5 +166,6 @@ def talking_heads_attention(q, k_cache, v_cache, talk, gate_pre, heads: int, kv_
     keys of each query into that many independent sweeps (decode over long caches)."""
     from ._native import native_seq, use_seq
     if use_seq(q):
-        return native_seq().talk_attention(q, k_cache, v_cache, talk, gate_pre, heads, kv_heads, scale, nsplit, sb.desc)
+        return native_seq().talk_attention(q, k_cache, v_cache, talk, gate_pre, heads, kv_heads, scale, nsplit, sb.desc,
+                                           sb.tiles)
     return ref.talk_attention(q, k_cache, v_cache, talk, gate_pre, heads, kv_heads, scale, sb)

@@ -400,3 +400,51 @@ def test_decode_graphs_replay_equals_eager():
         close(graph[k], eager[k].double(), 1e-5)
     close(eager["a"], O.forward(cfg, W, a[:29]))
     close(eager["c"], O.forward(cfg, W, c))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dk,dv,H,G", [(32, 32, 4, 2), (64, 128, 6, 3), (144, 160, 2, 1), (128, 64, 8, 8)])
+@pytest.mark.parametrize("scale", [0.2, 4.0])
+def test_matrix_core_attention_sweep(dk, dv, H, G, scale):
+    """bf16 head-mixing attention on the matrix-core kernel (ragged batch, continued sequences, tiles that end inside
+    a sequence, key splits) against per-query float64 sums over the same bf16 inputs; a sharp scale makes single keys
+    carry the result."""
+    from llm_in_practise_amd.models.common import SeqStateCache
+    from llm_in_practise_amd.ops.attention import talking_heads_attention
+    g = torch.Generator().manual_seed(dk + dv)
+    lens, starts, slots, max_len = [70, 1, 33, 32, 5], [0, 130, 31, 64, 0], [4, 0, 2, 5, 1], 256
+    cache = SeqStateCache([{"k": ((G * dk,), "kv"), "v": ((G * dv,), "kv")}], 6, max_len, torch.bfloat16, "cuda")
+    kc = torch.randn(6, max_len, G * dk, generator=g).to(torch.bfloat16)
+    vc = torch.randn(6, max_len, G * dv, generator=g).to(torch.bfloat16)
+    cache.layers[0]["k"].copy_(kc)
+    cache.layers[0]["v"].copy_(vc)
+    T = sum(lens)
+    q = torch.randn(T, H * dk, generator=g).to(torch.bfloat16)
+    gate = torch.randn(T, H * dv, generator=g).to(torch.bfloat16)
+    talk = (torch.eye(H) + 0.3 * torch.randn(H, H, generator=g)).float()
+    sb = SeqBatch.packed(cache, slots, lens, starts)
+    for nsplit in (1, 3):
+        got = talking_heads_attention(q.cuda(), cache.layers[0]["k"], cache.layers[0]["v"], talk.cuda(), gate.cuda(), H, G,
+                                      scale, sb, nsplit).float().cpu()
+        t = 0
+        for b, n in enumerate(lens):
+            for i in range(n):
+                L = starts[b] + i + 1
+                kk = kc[slots[b], :L].double().view(L, G, dk)
+                vv = vc[slots[b], :L].double().view(L, G, dv)
+                w = torch.stack([torch.softmax(kk[:, h // (H // G)] @ q[t].double().view(H, dk)[h] * scale, 0) for h in range(H)])
+                w = talk.double() @ w
+                o = torch.stack([w[h] @ vv[:, h // (H // G)] for h in range(H)]).reshape(-1) * torch.sigmoid(gate[t].double())
+                err = (got[t].double() - o).abs().max() / o.abs().max()
+                assert err < 2e-2, (b, i, nsplit, float(err))
+                t += 1
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_bf16_matrix_core_sizes_long_context(device):
+    """bf16 model whose attention sizes take the matrix-core path; 600 tokens, then decoding across key splits."""
+    cfg = config([parallel(lh=4, lg=2, ldim=32, lvdim=32, lconv=3, scale=0.25, mlp=None), mlstm()], width=64)
+    lm, W = build(cfg, device, seed=12, dtype=torch.bfloat16)
+    toks = tokens(620, cfg["vocab"], 19)
+    got = replay(lm, 1100, [([("a", toks[:600])], [])] + [([("a", [t])], []) for t in toks[600:]])["a"]
+    close(got, O.forward(cfg, W, toks), 0.06)
