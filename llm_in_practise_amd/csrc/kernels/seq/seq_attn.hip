@@ -83,7 +83,9 @@ __global__ __launch_bounds__(64) void k_talk_attn_partial(const T* __restrict__ 
 // K and Q operands are 16 B global loads (Q stays in registers).  Rows past the cache end are clamped: their weights
 // are 0.  Writes the same partial format as the scalar kernel: m, l per (token, g, split) and unnormalised U columns
 // [c*dv, (c+1)*dv).
-template <int NDS, int NDT>
+// HEADS = true is the decode form: a tile is ONE token and its "queries" are the H/G query heads that share kv head
+// blockIdx.y, so a key tile is loaded once for the whole group instead of once per head.
+template <int NDS, int NDT, bool HEADS>
 __global__ __launch_bounds__(64) void k_talk_attn_mfma(const bf16* __restrict__ q, int ldq, const bf16* __restrict__ kc,
                                                        const bf16* __restrict__ vc, float* __restrict__ pm,
                                                        float* __restrict__ pl, float* __restrict__ pu,
@@ -92,13 +94,15 @@ __global__ __launch_bounds__(64) void k_talk_attn_mfma(const bf16* __restrict__ 
                                                        float scale, SeqDesc d) {
   constexpr int LDMAX = NDT * 32 + 8;
   __shared__ __attribute__((aligned(16))) bf16 sV[32 * LDMAX];
-  const int tile = blockIdx.x, g = blockIdx.y, c = blockIdx.z % G, z = blockIdx.z / G;
-  const int lane = threadIdx.x, hi = lane >> 5, ql = lane & 31;
+  const int tile = blockIdx.x, c = blockIdx.z % G, z = blockIdx.z / G;
+  const int lane = threadIdx.x, hi = lane >> 5, ql = lane & 31, rep = H / G;
   const int s = tile_seq[tile], t0 = tile_t0[tile], tend = d.seq_off[s + 1], slot = d.slots[s];
-  const int tq = min(t0 + ql, tend - 1);
-  const bool valid_q = t0 + ql < tend;
-  const int pos_q = d.tok_pos[tq], pmax = d.tok_pos[min(t0 + 31, tend - 1)];
-  const int nds = dk >> 4, ndt = dv >> 5, LD = dv + 8, GV = G * dv, kh = g / (H / G);
+  const int tq = HEADS ? t0 : min(t0 + ql, tend - 1);
+  const int g = HEADS ? blockIdx.y * rep + min(ql, rep - 1) : blockIdx.y;
+  const bool valid_q = HEADS ? ql < rep : t0 + ql < tend;
+  const int pos_q = d.tok_pos[tq], pmax = HEADS ? pos_q : d.tok_pos[min(t0 + 31, tend - 1)];
+  const int nds = dk >> 4, ndt = dv >> 5, LD = dv + 8, GV = G * dv, kh = HEADS ? blockIdx.y : g / rep;
+  const float sl2 = scale * 1.4426950408889634f;   // scores in units of log2: v_exp_f32 is 2^x
   const int per = (pmax + nsplit) / nsplit, j0 = z * per, j1 = min(pmax + 1, j0 + per);
   const bf16* kbase = kc + ((size_t)slot * max_len) * (G * dk) + kh * dk + 8 * hi;
   const bf16* vbase = vc + ((size_t)slot * max_len) * GV + c * dv;
@@ -132,16 +136,16 @@ __global__ __launch_bounds__(64) void k_talk_attn_mfma(const bf16* __restrict__ 
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       const int key = jb + (r & 3) + 8 * (r >> 2) + 4 * hi;
-      sc[r] = (key <= pos_q && key < j1) ? sc[r] * scale : -INFINITY;
+      sc[r] = (key <= pos_q && key < j1) ? sc[r] * sl2 : -INFINITY;
       mt = fmaxf(mt, sc[r]);
     }
     mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
     const float mn = fmaxf(m, mt), ms = mn == -INFINITY ? 0.f : mn;
-    const float corr = expf(m - ms);
+    const float corr = __builtin_amdgcn_exp2f(m - ms);
     float rs = 0.f;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-      sc[r] = expf(sc[r] - ms);
+      sc[r] = __builtin_amdgcn_exp2f(sc[r] - ms);
       rs += sc[r];
     }
     rs += __shfl_xor(rs, 32, 64);
@@ -173,7 +177,7 @@ __global__ __launch_bounds__(64) void k_talk_attn_mfma(const bf16* __restrict__ 
   if (!valid_q) return;
   const size_t o = ((size_t)tq * H + g) * nsplit + z;
   if (c == 0 && hi == 0) {
-    pm[o] = m;
+    pm[o] = m * 0.6931471805599453f;             // back to natural units, as the scalar sweep writes them
     pl[o] = l;
   }
 #pragma unroll
@@ -185,32 +189,48 @@ __global__ __launch_bounds__(64) void k_talk_attn_mfma(const bf16* __restrict__ 
             f32x4{acc[dt][4 * r4], acc[dt][4 * r4 + 1], acc[dt][4 * r4 + 2], acc[dt][4 * r4 + 3]};
 }
 
-// out[t, h, c] = sigmoid(gate[t, h*dv + c]) * sum_g talk[h, g] * U_g[kv(h)*dv + c] / l_g   (splits merged first)
+// Pass 2.  One block per (token, 64 value columns of one kv head c): first the splits of every query head g are
+// merged and normalised into LDS, L[g][col] = sum_z e_z U_gz[col] / sum_z e_z l_gz with e_z = exp(m_gz - max_z m_gz);
+// then every output head h of kv head c takes out[h][col] = sigmoid(gate) * sum_g talk[h][g] L[g][col].
+constexpr int MH = 128;    // query heads held in LDS
 template <typename T>
-__global__ __launch_bounds__(64) void k_talk_attn_merge(const float* __restrict__ pm, const float* __restrict__ pl,
-                                                        const float* __restrict__ pu, const float* __restrict__ talk,
-                                                        const T* __restrict__ gate, int ldg, T* __restrict__ out, int H,
-                                                        int G, int dv, int nsplit) {
-  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-  const int kh = h / (H / G), GV = G * dv;
-  for (int c = lane; c < dv; c += 64) {
-    float o = 0.f;
-    for (int g = 0; g < H; ++g) {
-      const size_t b = ((size_t)t * H + g) * nsplit;
-      float mx = -INFINITY;
-      for (int z = 0; z < nsplit; ++z) mx = fmaxf(mx, pm[b + z]);
-      float l = 0.f, u = 0.f;
-      for (int z = 0; z < nsplit; ++z) {
-        const float e = expf(pm[b + z] - mx);
-        l += e * pl[b + z];
-        u += e * pu[(b + z) * GV + kh * dv + c];
-      }
-      o += talk[h * H + g] * (u / l);
+__global__ __launch_bounds__(256) void k_talk_attn_merge(const float* __restrict__ pm, const float* __restrict__ pl,
+                                                         const float* __restrict__ pu, const float* __restrict__ talk,
+                                                         const T* __restrict__ gate, int ldg, T* __restrict__ out, int H,
+                                                         int G, int dv, int nsplit) {
+  extern __shared__ float L[];                     // [H][64]
+  const int t = blockIdx.x, nch = (dv + 63) / 64, c = blockIdx.y / nch, ch = blockIdx.y % nch;
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, col = ch * 64 + lane, GV = G * dv, rep = H / G;
+  for (int g = w; g < H; g += 4) {
+    const size_t b = ((size_t)t * H + g) * nsplit;
+    float mx = -INFINITY;
+    for (int z = 0; z < nsplit; ++z) mx = fmaxf(mx, pm[b + z]);
+    float l = 0.f, u = 0.f;
+    for (int z = 0; z < nsplit; ++z) {
+      const float e = expf(pm[b + z] - mx);
+      l += e * pl[b + z];
+      if (col < dv) u += e * pu[(b + z) * GV + c * dv + col];
     }
-    out[(size_t)t * (H * dv) + h * dv + c] = (T)(o * sigmoidf_((float)gate[(size_t)t * ldg + h * dv + c]));
+    L[g * 64 + lane] = u / l;
+  }
+  __syncthreads();
+  if (col >= dv) return;
+  for (int hl = w; hl < rep; hl += 4) {
+    const int h = c * rep + hl;
+    float o = 0.f;
+    for (int g = 0; g < H; ++g) o += talk[h * H + g] * L[g * 64 + lane];
+    out[(size_t)t * (H * dv) + h * dv + col] = (T)(o * sigmoidf_((float)gate[(size_t)t * ldg + h * dv + col]));
   }
 }
 
+template <typename T>
+static void launch_merge(const float* pm, const float* pl, const float* pu, const float* talk, const T* gate, int ldg,
+                         T* out, int Ttot, int H, int G, int dv, int nsplit, hipStream_t st) {
+  hipLaunchKernelGGL(k_talk_attn_merge<T>, dim3(Ttot, G * ((dv + 63) / 64)), dim3(256), sizeof(float) * H * 64, st, pm,
+                     pl, pu, talk, gate, ldg, out, H, G, dv, nsplit);
+}
+
+int seq_attn_max_heads() { return MH; }
 int seq_attn_max_cols() { return 64 * MAXC; }
 
 // the MFMA sweep needs bf16, 16-byte rows and whole operand tiles
@@ -224,23 +244,25 @@ void seq_talk_attention(int code, const void* q, int ldq, const void* kc, const 
                         SeqDesc d, hipStream_t st) {
   if (d.Ttot == 0) return;
   if (tile_seq != nullptr && seq_attn_mfma_ok(code, ldq, dk, dv)) {
-    const dim3 grid(ntiles, H, G * nsplit);
-    if (dk <= 128 && dv <= 128)
-      hipLaunchKernelGGL((k_talk_attn_mfma<8, 4>), grid, dim3(64), 0, st, (const bf16*)q, ldq, (const bf16*)kc,
-                         (const bf16*)vc, pm, pl, pu, tile_seq, tile_t0, H, G, dk, dv, max_len, nsplit, scale, d);
-    else
-      hipLaunchKernelGGL((k_talk_attn_mfma<16, 8>), grid, dim3(64), 0, st, (const bf16*)q, ldq, (const bf16*)kc,
-                         (const bf16*)vc, pm, pl, pu, tile_seq, tile_t0, H, G, dk, dv, max_len, nsplit, scale, d);
-    hipLaunchKernelGGL(k_talk_attn_merge<bf16>, dim3(d.Ttot, H), dim3(64), 0, st, pm, pl, pu, talk, (const bf16*)gate,
-                       ldg, (bf16*)out, H, G, dv, nsplit);
+    const bool heads = ntiles == d.Ttot && H / G <= 32 && H / G > 1;    // one token per tile: group the heads instead
+    const dim3 grid(ntiles, heads ? G : H, G * nsplit);
+#define SEQ_ATTN_LAUNCH(NDS, NDT, HEADS)                                                                              \
+  hipLaunchKernelGGL((k_talk_attn_mfma<NDS, NDT, HEADS>), grid, dim3(64), 0, st, (const bf16*)q, ldq, (const bf16*)kc, \
+                     (const bf16*)vc, pm, pl, pu, tile_seq, tile_t0, H, G, dk, dv, max_len, nsplit, scale, d)
+    if (dk <= 128 && dv <= 128) {
+      if (heads) SEQ_ATTN_LAUNCH(8, 4, true); else SEQ_ATTN_LAUNCH(8, 4, false);
+    } else {
+      if (heads) SEQ_ATTN_LAUNCH(16, 8, true); else SEQ_ATTN_LAUNCH(16, 8, false);
+    }
+#undef SEQ_ATTN_LAUNCH
+    launch_merge<bf16>(pm, pl, pu, talk, (const bf16*)gate, ldg, (bf16*)out, d.Ttot, H, G, dv, nsplit, st);
     LIPA_CHECK_LAUNCH();
     return;
   }
   SEQ_DISPATCH_T(code, {
     hipLaunchKernelGGL(k_talk_attn_partial<T>, dim3(d.Ttot, H, nsplit), dim3(64), sizeof(float) * dk, st, (const T*)q,
                        ldq, (const T*)kc, (const T*)vc, pm, pl, pu, H, G, dk, dv, max_len, nsplit, scale, d);
-    hipLaunchKernelGGL(k_talk_attn_merge<T>, dim3(d.Ttot, H), dim3(64), 0, st, pm, pl, pu, talk, (const T*)gate, ldg,
-                       (T*)out, H, G, dv, nsplit);
+    launch_merge<T>(pm, pl, pu, talk, (const T*)gate, ldg, (T*)out, d.Ttot, H, G, dv, nsplit, st);
   });
   LIPA_CHECK_LAUNCH();
 }

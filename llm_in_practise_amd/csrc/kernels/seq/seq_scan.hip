@@ -2,12 +2,13 @@
 // maximum; gated delta rule with a per-channel decay), over packed variable-length sequences with per-slot state.
 //
 // Recurrences: every column of the state matrix S[dk, dv] evolves on its own given the step's k, q and gates, so a
-// block owns one (sequence, head) and up to 256/R columns; a column's dk rows are spread over R adjacent lanes
-// (R a power of two <= 64, <= 16 rows per lane, rows interleaved i*R + rg) and live in registers for the whole
-// scan.  Dot products over dk are finished with xor-shuffles inside the R-lane group: no barrier per token.  The
-// step inputs of 16 tokens at a time are staged through LDS as float.  One token is the decode step: load state,
-// one update, store.  State layout in HBM: S [slots, H, dv, dk] (a lane's rows are R apart, a group's lanes
-// adjacent: coalesced), float.
+// block owns one (sequence, head) and 256/R columns; a column's dk rows are spread over R adjacent lanes (R a power
+// of two <= 16, a template parameter; 16 contiguous rows per lane) and live in registers for the whole scan.  Dot
+// products over dk run as four independent partial sums per lane and are finished with constant-mask xor-shuffles
+// inside the R-lane group: no barrier per token.  The step inputs of 16 tokens at a time are staged through LDS as
+// float rows of 16*R entries, zero-padded past dk (a padded row never changes: k = 0), and read back as 16-byte
+// vectors.  One token is the decode step: load state, one update, store.  State layout in HBM: S [slots, H, dv, dk],
+// float.
 #include "seq_common.h"
 
 using namespace lipa;
@@ -105,48 +106,89 @@ __global__ __launch_bounds__(256) void k_conv_state(const T* __restrict__ u, int
     if (i < taps - 1) state[((size_t)slot * (taps - 1) + i) * C + ch] = (T)nv[i];
 }
 
-__device__ __forceinline__ float group_sum(float v, int R) {
-  for (int o = R >> 1; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+// sum over the R adjacent lanes of a group (R <= 16, groups aligned inside a 16-lane row) with data-parallel
+// primitives only: swap inside pairs, swap pairs inside quads, mirror the half row, mirror the row.  After each step
+// every lane of the widened group holds the same partial sum, so a mirror pairs equal-valued halves.
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float v) {
+  return v + __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), CTRL, 0xF, 0xF, true));
+}
+template <int R>
+__device__ __forceinline__ float group_sum(float v) {
+  if (R >= 2) v = dpp_add<0xB1>(v);    // quad_perm [1, 0, 3, 2]
+  if (R >= 4) v = dpp_add<0x4E>(v);    // quad_perm [2, 3, 0, 1]
+  if (R >= 8) v = dpp_add<0x141>(v);   // row_half_mirror
+  if (R >= 16) v = dpp_add<0x140>(v);  // row_mirror
   return v;
+}
+
+// a lane's 16 contiguous state rows: 16-byte accesses when the row length allows
+__device__ __forceinline__ void load_rows(const float* p, int r0, int dk, bool on, float (&r)[KR]) {
+  if (on && (dk & 3) == 0) {
+#pragma unroll
+    for (int i4 = 0; i4 < KR / 4; ++i4) {
+      f32x4 v = {0.f, 0.f, 0.f, 0.f};
+      if (r0 + 4 * i4 < dk) v = *reinterpret_cast<const f32x4*>(p + r0 + 4 * i4);
+      r[4 * i4] = v[0]; r[4 * i4 + 1] = v[1]; r[4 * i4 + 2] = v[2]; r[4 * i4 + 3] = v[3];
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < KR; ++i) r[i] = (on && r0 + i < dk) ? p[r0 + i] : 0.f;
+  }
+}
+__device__ __forceinline__ void store_rows(float* p, int r0, int dk, const float (&r)[KR]) {
+  if ((dk & 3) == 0) {
+#pragma unroll
+    for (int i4 = 0; i4 < KR / 4; ++i4)
+      if (r0 + 4 * i4 < dk)
+        *reinterpret_cast<f32x4*>(p + r0 + 4 * i4) = f32x4{r[4 * i4], r[4 * i4 + 1], r[4 * i4 + 2], r[4 * i4 + 3]};
+  } else {
+#pragma unroll
+    for (int i = 0; i < KR; ++i)
+      if (r0 + i < dk) p[r0 + i] = r[i];
+  }
+}
+
+// stage n tokens of a [*, ld] matrix's dk columns at `col0` into LDS rows of DKP floats (zero / `pad` past dk)
+template <typename T, int DKP>
+__device__ __forceinline__ void stage_rows(float* dst, const T* __restrict__ src, size_t ld, int col0, int dk, int n,
+                                           float mul, float pad) {
+  for (int e = threadIdx.x; e < n * DKP; e += 256) {
+    const int tt = e / DKP, r = e % DKP;
+    dst[e] = r < dk ? (float)src[(size_t)tt * ld + col0 + r] * mul : pad;
+  }
 }
 
 // mLSTM.  m_t = max(f + m, i); S = e^(f+m-m_t) S + e^(i-m_t) k v^T; n likewise; o = S^T q / (max(|n.q|, e^-m_t) + 1e-6)
 // with i = cap tanh((ipre + ib) / cap), f = logsigmoid(cap tanh((fpre + fb) / cap)); m starts at 0.
-template <typename T>
+template <typename T, int R>
 __global__ __launch_bounds__(256) void k_mlstm_scan(const T* __restrict__ q, int ldq, const T* __restrict__ k, int ldk,
                                                     const T* __restrict__ v, int ldv, const float* __restrict__ ipre,
                                                     const float* __restrict__ fpre, const float* __restrict__ ib,
                                                     const float* __restrict__ fb, float cap, float qscale,
                                                     float* __restrict__ S, float* __restrict__ N, float* __restrict__ M,
-                                                    float* __restrict__ out, int H, int dk, int dv, int R, SeqDesc d) {
-  extern __shared__ float smem[];
+                                                    float* __restrict__ out, int H, int dk, int dv, SeqDesc d) {
+  constexpr int DKP = KR * R, NC = 256 / R;
+  __shared__ __attribute__((aligned(16))) float sk[CT * DKP];
+  __shared__ __attribute__((aligned(16))) float sq[CT * DKP];
+  __shared__ float sv[CT * NC];
+  __shared__ float sg[2 * CT];
   const int s = blockIdx.x / H, hd = blockIdx.x % H, cb = blockIdx.y, tid = threadIdx.x;
   if (d.live && !d.live[s]) return;
-  const int NC = 256 / R, rg = tid % R, cl = tid / R, col = cb * NC + cl;
+  const int rg = tid % R, cl = tid / R, col = cb * NC + cl, r0 = rg * KR;
   const bool colok = col < dv;
   const int t0 = d.seq_off[s], t1 = d.seq_off[s + 1], p0 = d.pos0[s], slot = d.slots[s];
-  float* sk = smem;
-  float* sq = sk + CT * dk;
-  float* sv = sq + CT * dk;
-  float* sg = sv + CT * NC;
   const size_t hbase = (size_t)slot * H + hd;
   float* Sp = S + (hbase * dv + (colok ? col : 0)) * dk;
   float Sr[KR], nr[KR];
   float m = p0 > 0 ? M[hbase] : 0.f;
-#pragma unroll
-  for (int i = 0; i < KR; ++i) {
-    const int row = i * R + rg;
-    Sr[i] = (p0 > 0 && colok && row < dk) ? Sp[row] : 0.f;
-    nr[i] = (p0 > 0 && row < dk) ? N[hbase * dk + row] : 0.f;
-  }
+  load_rows(Sp, r0, dk, p0 > 0 && colok, Sr);
+  load_rows(N + hbase * dk, r0, dk, p0 > 0, nr);
   for (int c0 = t0; c0 < t1; c0 += CT) {
     const int n = min(CT, t1 - c0);
     __syncthreads();
-    for (int e = tid; e < n * dk; e += 256) {
-      const int tt = e / dk, r = e % dk;
-      sk[e] = (float)k[(size_t)(c0 + tt) * ldk + hd * dk + r];
-      sq[e] = (float)q[(size_t)(c0 + tt) * ldq + hd * dk + r] * qscale;
-    }
+    stage_rows<T, DKP>(sk, k + (size_t)c0 * ldk, ldk, hd * dk, dk, n, 1.f, 0.f);
+    stage_rows<T, DKP>(sq, q + (size_t)c0 * ldq, ldq, hd * dk, dk, n, qscale, 0.f);
     for (int e = tid; e < n * NC; e += 256) {
       const int tt = e / NC, cc = cb * NC + e % NC;
       sv[e] = cc < dv ? (float)v[(size_t)(c0 + tt) * ldv + hd * dv + cc] : 0.f;
@@ -163,69 +205,58 @@ __global__ __launch_bounds__(256) void k_mlstm_scan(const T* __restrict__ q, int
       const float a = expf(fg + m - mn), b = expf(ig - mn);
       m = mn;
       const float bv = b * sv[tt * NC + cl];
-      float num = 0.f, den = 0.f;
+      float num[4] = {0.f, 0.f, 0.f, 0.f}, den[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int i = 0; i < KR; ++i) {
-        const int row = i * R + rg;
-        const bool ok = row < dk;
-        const float kk = ok ? sk[tt * dk + row] : 0.f, qq = ok ? sq[tt * dk + row] : 0.f;
-        Sr[i] = a * Sr[i] + kk * bv;
-        nr[i] = a * nr[i] + b * kk;
-        num += Sr[i] * qq;
-        den += nr[i] * qq;
+      for (int i4 = 0; i4 < KR / 4; ++i4) {
+        const f32x4 kk = *reinterpret_cast<const f32x4*>(sk + tt * DKP + r0 + 4 * i4);
+        const f32x4 qq = *reinterpret_cast<const f32x4*>(sq + tt * DKP + r0 + 4 * i4);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int i = 4 * i4 + j;
+          Sr[i] = a * Sr[i] + kk[j] * bv;
+          nr[i] = a * nr[i] + b * kk[j];
+          num[j] += Sr[i] * qq[j];
+          den[j] += nr[i] * qq[j];
+        }
       }
-      num = group_sum(num, R);
-      den = group_sum(den, R);
+      const float nm = group_sum<R>((num[0] + num[1]) + (num[2] + num[3]));
+      const float dn = group_sum<R>((den[0] + den[1]) + (den[2] + den[3]));
       if (rg == 0 && colok)
-        out[((size_t)(c0 + tt) * H + hd) * dv + col] = num / (fmaxf(fabsf(den), expf(-m)) + 1e-6f);
+        out[((size_t)(c0 + tt) * H + hd) * dv + col] = nm / (fmaxf(fabsf(dn), expf(-m)) + 1e-6f);
     }
   }
-#pragma unroll
-  for (int i = 0; i < KR; ++i) {
-    const int row = i * R + rg;
-    if (row < dk) {
-      if (colok) Sp[row] = Sr[i];
-      if (cb == 0 && cl == 0) N[hbase * dk + row] = nr[i];
-    }
-  }
+  if (colok) store_rows(Sp, r0, dk, Sr);
+  if (cb == 0 && cl == 0) store_rows(N + hbase * dk, r0, dk, nr);
   if (cb == 0 && tid == 0) M[hbase] = m;
 }
 
 // Gated delta rule.  S <- g * S (g per key channel); u = beta (v - S^T k); S <- S + k u^T; o = S^T q.
 // beta = sigmoid(bpre); head hd reads q/k head hd / (H / G).
-template <typename T>
+template <typename T, int R>
 __global__ __launch_bounds__(256) void k_delta_scan(const T* __restrict__ q, int ldq, const T* __restrict__ k, int ldk,
                                                     const T* __restrict__ v, int ldv, const float* __restrict__ g,
                                                     const float* __restrict__ bpre, float* __restrict__ S,
-                                                    float* __restrict__ out, int H, int G, int dk, int dv, int R,
-                                                    SeqDesc d) {
-  extern __shared__ float smem[];
+                                                    float* __restrict__ out, int H, int G, int dk, int dv, SeqDesc d) {
+  constexpr int DKP = KR * R, NC = 256 / R;
+  __shared__ __attribute__((aligned(16))) float sk[CT * DKP];
+  __shared__ __attribute__((aligned(16))) float sq[CT * DKP];
+  __shared__ __attribute__((aligned(16))) float sd[CT * DKP];
+  __shared__ float sv[CT * NC];
+  __shared__ float sb[CT];
   const int s = blockIdx.x / H, hd = blockIdx.x % H, cb = blockIdx.y, tid = threadIdx.x;
   if (d.live && !d.live[s]) return;
-  const int NC = 256 / R, rg = tid % R, cl = tid / R, col = cb * NC + cl, kh = hd / (H / G);
+  const int rg = tid % R, cl = tid / R, col = cb * NC + cl, kh = hd / (H / G), r0 = rg * KR;
   const bool colok = col < dv;
   const int t0 = d.seq_off[s], t1 = d.seq_off[s + 1], p0 = d.pos0[s], slot = d.slots[s];
-  float* sk = smem;
-  float* sq = sk + CT * dk;
-  float* sd = sq + CT * dk;
-  float* sv = sd + CT * dk;
-  float* sb = sv + CT * NC;
   float* Sp = S + (((size_t)slot * H + hd) * dv + (colok ? col : 0)) * dk;
   float Sr[KR];
-#pragma unroll
-  for (int i = 0; i < KR; ++i) {
-    const int row = i * R + rg;
-    Sr[i] = (p0 > 0 && colok && row < dk) ? Sp[row] : 0.f;
-  }
+  load_rows(Sp, r0, dk, p0 > 0 && colok, Sr);
   for (int c0 = t0; c0 < t1; c0 += CT) {
     const int n = min(CT, t1 - c0);
     __syncthreads();
-    for (int e = tid; e < n * dk; e += 256) {
-      const int tt = e / dk, r = e % dk;
-      sk[e] = (float)k[(size_t)(c0 + tt) * ldk + kh * dk + r];
-      sq[e] = (float)q[(size_t)(c0 + tt) * ldq + kh * dk + r];
-      sd[e] = g[((size_t)(c0 + tt) * H + hd) * dk + r];
-    }
+    stage_rows<T, DKP>(sk, k + (size_t)c0 * ldk, ldk, kh * dk, dk, n, 1.f, 0.f);
+    stage_rows<T, DKP>(sq, q + (size_t)c0 * ldq, ldq, kh * dk, dk, n, 1.f, 0.f);
+    stage_rows<float, DKP>(sd, g + (size_t)c0 * H * dk, (size_t)H * dk, hd * dk, dk, n, 1.f, 1.f);
     for (int e = tid; e < n * NC; e += 256) {
       const int tt = e / NC, cc = cb * NC + e % NC;
       sv[e] = cc < dv ? (float)v[(size_t)(c0 + tt) * ldv + hd * dv + cc] : 0.f;
@@ -233,35 +264,34 @@ __global__ __launch_bounds__(256) void k_delta_scan(const T* __restrict__ q, int
     if (tid < n) sb[tid] = sigmoidf_(bpre[(size_t)(c0 + tid) * H + hd]);
     __syncthreads();
     for (int tt = 0; tt < n; ++tt) {
-      float dot = 0.f;
+      f32x4 kk[KR / 4];
+      float dot[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int i = 0; i < KR; ++i) {
-        const int row = i * R + rg;
-        if (row < dk) {
-          Sr[i] *= sd[tt * dk + row];
-          dot += Sr[i] * sk[tt * dk + row];
+      for (int i4 = 0; i4 < KR / 4; ++i4) {
+        kk[i4] = *reinterpret_cast<const f32x4*>(sk + tt * DKP + r0 + 4 * i4);
+        const f32x4 gd = *reinterpret_cast<const f32x4*>(sd + tt * DKP + r0 + 4 * i4);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          Sr[4 * i4 + j] *= gd[j];
+          dot[j] += Sr[4 * i4 + j] * kk[i4][j];
         }
       }
-      dot = group_sum(dot, R);
-      const float u = sb[tt] * (sv[tt * NC + cl] - dot);
-      float o = 0.f;
+      const float u = sb[tt] * (sv[tt * NC + cl] - group_sum<R>((dot[0] + dot[1]) + (dot[2] + dot[3])));
+      float o[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int i = 0; i < KR; ++i) {
-        const int row = i * R + rg;
-        if (row < dk) {
-          Sr[i] += sk[tt * dk + row] * u;
-          o += Sr[i] * sq[tt * dk + row];
+      for (int i4 = 0; i4 < KR / 4; ++i4) {
+        const f32x4 qq = *reinterpret_cast<const f32x4*>(sq + tt * DKP + r0 + 4 * i4);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          Sr[4 * i4 + j] += kk[i4][j] * u;
+          o[j] += Sr[4 * i4 + j] * qq[j];
         }
       }
-      o = group_sum(o, R);
-      if (rg == 0 && colok) out[((size_t)(c0 + tt) * H + hd) * dv + col] = o;
+      const float ov = group_sum<R>((o[0] + o[1]) + (o[2] + o[3]));
+      if (rg == 0 && colok) out[((size_t)(c0 + tt) * H + hd) * dv + col] = ov;
     }
   }
-#pragma unroll
-  for (int i = 0; i < KR; ++i) {
-    const int row = i * R + rg;
-    if (row < dk && colok) Sp[row] = Sr[i];
-  }
+  if (colok) store_rows(Sp, r0, dk, Sr);
 }
 
 // ---------------------------------------------------------------------------------------------- launchers
@@ -271,9 +301,18 @@ static int rows_split(int dk) {
   return R;
 }
 
-int seq_scan_max_dk() { return 256; }   // 3 staged arrays of CT x dk floats stay under 64 KB of LDS
+int seq_scan_max_dk() { return KR * 16; }
 int seq_conv_max_head() { return 64 * MAXHW; }
 int seq_conv_max_taps() { return MAXTAPS; }
+
+#define SEQ_DISPATCH_R(R_, ...)                          \
+  switch (R_) {                                          \
+    case 1: { constexpr int R = 1; __VA_ARGS__; } break; \
+    case 2: { constexpr int R = 2; __VA_ARGS__; } break; \
+    case 4: { constexpr int R = 4; __VA_ARGS__; } break; \
+    case 8: { constexpr int R = 8; __VA_ARGS__; } break; \
+    default: { constexpr int R = 16; __VA_ARGS__; } break; \
+  }
 
 // segs: nseg x {c0, nheads, hw, mode}; sw: nseg norm-weight pointers (or null); sscale: nseg scales
 void seq_short_conv(int code, int out_f32, const void* u, int ldu, const float* w, void* state, void* out, int C,
@@ -305,21 +344,23 @@ void seq_mlstm_scan(int code, const void* q, int ldq, const void* k, int ldk, co
                     const float* fpre, const float* ib, const float* fb, float cap, float qscale, float* S, float* N,
                     float* M, float* out, int H, int dk, int dv, SeqDesc d, hipStream_t st) {
   if (d.B == 0) return;
-  const int R = rows_split(dk), NC = 256 / R;
-  const size_t lds = sizeof(float) * ((size_t)2 * CT * dk + CT * NC + 2 * CT);
-  SEQ_DISPATCH_T(code, hipLaunchKernelGGL(k_mlstm_scan<T>, dim3(d.B * H, (dv + NC - 1) / NC), dim3(256), lds, st,
-                                          (const T*)q, ldq, (const T*)k, ldk, (const T*)v, ldv, ipre, fpre, ib, fb, cap,
-                                          qscale, S, N, M, out, H, dk, dv, R, d));
+  const int Rr = rows_split(dk);
+  SEQ_DISPATCH_T(code, SEQ_DISPATCH_R(Rr, {
+    constexpr int NC = 256 / R;
+    hipLaunchKernelGGL((k_mlstm_scan<T, R>), dim3(d.B * H, (dv + NC - 1) / NC), dim3(256), 0, st, (const T*)q, ldq,
+                       (const T*)k, ldk, (const T*)v, ldv, ipre, fpre, ib, fb, cap, qscale, S, N, M, out, H, dk, dv, d);
+  }));
   LIPA_CHECK_LAUNCH();
 }
 
 void seq_delta_scan(int code, const void* q, int ldq, const void* k, int ldk, const void* v, int ldv, const float* g,
                     const float* bpre, float* S, float* out, int H, int G, int dk, int dv, SeqDesc d, hipStream_t st) {
   if (d.B == 0) return;
-  const int R = rows_split(dk), NC = 256 / R;
-  const size_t lds = sizeof(float) * ((size_t)3 * CT * dk + CT * NC + CT);
-  SEQ_DISPATCH_T(code, hipLaunchKernelGGL(k_delta_scan<T>, dim3(d.B * H, (dv + NC - 1) / NC), dim3(256), lds, st,
-                                          (const T*)q, ldq, (const T*)k, ldk, (const T*)v, ldv, g, bpre, S, out, H, G,
-                                          dk, dv, R, d));
+  const int Rr = rows_split(dk);
+  SEQ_DISPATCH_T(code, SEQ_DISPATCH_R(Rr, {
+    constexpr int NC = 256 / R;
+    hipLaunchKernelGGL((k_delta_scan<T, R>), dim3(d.B * H, (dv + NC - 1) / NC), dim3(256), 0, st, (const T*)q, ldq,
+                       (const T*)k, ldk, (const T*)v, ldv, g, bpre, S, out, H, G, dk, dv, d);
+  }));
   LIPA_CHECK_LAUNCH();
 }

@@ -42,6 +42,7 @@ int seq_scan_max_dk();
 int seq_conv_max_head();
 int seq_conv_max_taps();
 int seq_attn_max_cols();
+int seq_attn_max_heads();
 
 using at::Tensor;
 using c10::optional;
@@ -296,6 +297,7 @@ Tensor talk_attention(Tensor q, Tensor kc, Tensor vc, Tensor talk, Tensor gate, 
               "value cache: [slots, max_len, G * dv]");
   const int64_t dv = vc.size(2) / G, max_len = kc.size(1);
   TORCH_CHECK(G * dv <= seq_attn_max_cols(), "attention: G * dv above ", seq_attn_max_cols());
+  TORCH_CHECK(H <= seq_attn_max_heads(), "attention: more than ", seq_attn_max_heads(), " heads");
   TORCH_CHECK(nsplit >= 1 && nsplit <= 1024, "nsplit");
   f32c(talk, "talk");
   TORCH_CHECK(talk.numel() == H * H, "talk: [H, H]");

@@ -311,7 +311,7 @@ class MobupelModel(nn.Module):
 
     def make_cache(self, batch: int, max_len: int, device=None) -> SeqStateCache:
         cache = SeqStateCache(self.state_specs(), batch, max_len, self.dtype, device or self.embed_tokens.device)
-        cache.decode_splits = max(1, min(16, max_len // 512))     # key splits of decode attention: fixed per cache
+        cache.decode_splits = max(1, min(32, max_len // 128))     # key splits of decode attention: fixed per cache
         return cache
 
     def run(self, tokens: torch.Tensor, sb: SeqBatch) -> torch.Tensor:
