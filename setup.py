@@ -11,8 +11,9 @@ from setuptools.command.build_ext import build_ext as _build_ext
 
 class build_ext(_build_ext):
     def run(self):
-        from llm_in_practise_amd.csrc.build import build_cpu_extension, build_hip_extension
+        from llm_in_practise_amd.csrc.build import build_cpu_extension, build_hip_extension, build_seq_extension
         build_hip_extension()
+        build_seq_extension()
         build_cpu_extension()
 
 
