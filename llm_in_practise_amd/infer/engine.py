@@ -633,16 +633,18 @@ class ServingEngine:
         active = [i for i, s in enumerate(self.slots) if s is not None]
         free = [i for i, s in enumerate(self.slots) if s is None]
         new = []
-        block = not active
+        block = idle = not active
         budget = self.prefill_token_budget
         while free and len(new) < self.max_prefill_batch:
             if self._held is not None:
                 r, self._held = self._held, None
             else:
                 try:
-                    # idle TP ranks wait inside a collective: heartbeat once a second
-                    tmo = (1.0 if self.tp_group is not None else None) if block else 0
-                    r = self.q.get(block=block, timeout=tmo)
+                    # idle TP ranks wait inside a collective: heartbeat once a second.  An idle engine that was just
+                    # woken by the first request of a burst gathers the rest of it (2 ms without a new arrival ends
+                    # the wait), so the burst is one packed prefill however the submitting thread is scheduled
+                    tmo = (1.0 if self.tp_group is not None else None) if block else (0.002 if idle else 0)
+                    r = self.q.get(block=block or idle, timeout=tmo)
                 except queue.Empty:
                     break
             block = False

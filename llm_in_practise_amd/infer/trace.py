@@ -36,7 +36,7 @@ class TraceRunner:
         if e is None or sum(s is None for s in e.slots) < need:
             if self.slot_of:
                 raise RuntimeError("a batch may grow only while no request is live")
-            slots = max(need, 2 * e.max_batch if e is not None else 1)
+            slots = max(2 * need, 2 * e.max_batch if e is not None else 8)     # room for a later, larger batch
             self.engine = e = ServingEngine(self.lm, None, max_batch=slots, max_model_len=self.max_len,
                                             use_graphs=self.use_graphs, start=False)
         return e
