@@ -79,30 +79,40 @@ __global__ __launch_bounds__(64) void k_talk_attn_partial(const T* __restrict__ 
 // split).  Scores are computed transposed, S^T[key][query] = K Q^T with v_mfma_f32_32x32x16_bf16: a lane then owns one
 // query (lane % 32) and 16 of the tile's 32 keys, so the softmax statistics are lane-local plus one exchange between
 // the wave's halves, and the weights P^T are already laid out as the B operand of O^T[col][query] += V^T P^T.  The
-// value tile goes through LDS row-major (16 B stores); a lane picks its column's 8 keys of a step with 2-byte reads.
+// value tile goes through LDS row-major (16 B stores); a lane gets its column's 8 keys of a step with two transposing
+// LDS reads (ds_read_tr16_b64).
 // K and Q operands are 16 B global loads (Q stays in registers).  Rows past the cache end are clamped: their weights
 // are 0.  Writes the same partial format as the scalar kernel: m, l per (token, g, split) and unnormalised U columns
 // [c*dv, (c+1)*dv).
 // HEADS = true is the decode form: a tile is ONE token and its "queries" are the H/G query heads that share kv head
 // blockIdx.y, so a key tile is loaded once for the whole group instead of once per head.
-template <int NDS, int NDT, bool HEADS>
-__global__ __launch_bounds__(64) void k_talk_attn_mfma(const bf16* __restrict__ q, int ldq, const bf16* __restrict__ kc,
+typedef __attribute__((address_space(3))) bf16x4 lds_bf16x4;
+__device__ __forceinline__ bf16x4 tr_read(const bf16* p) {
+  return __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_bf16x4*)(p));
+}
+
+// NW = 4 puts four query heads of one kv head (and one value head c) into a block: the key and value tiles are loaded
+// once into LDS for the four waves instead of once per head.
+template <int NDS, int NDT, bool HEADS, int NW>
+__global__ __launch_bounds__(64 * NW) void k_talk_attn_mfma(const bf16* __restrict__ q, int ldq, const bf16* __restrict__ kc,
                                                        const bf16* __restrict__ vc, float* __restrict__ pm,
                                                        float* __restrict__ pl, float* __restrict__ pu,
                                                        const int* __restrict__ tile_seq, const int* __restrict__ tile_t0,
                                                        int H, int G, int dk, int dv, int max_len, int nsplit,
                                                        float scale, SeqDesc d) {
-  constexpr int LDMAX = NDT * 32 + 8;
+  constexpr int LDMAX = NDT * 32 + 8, LDKMAX = NDS * 16 + 8;
   __shared__ __attribute__((aligned(16))) bf16 sV[32 * LDMAX];
+  __shared__ __attribute__((aligned(16))) bf16 sK[NW > 1 ? 32 * LDKMAX : 8];
   const int tile = blockIdx.x, c = blockIdx.z % G, z = blockIdx.z / G;
-  const int lane = threadIdx.x, hi = lane >> 5, ql = lane & 31, rep = H / G;
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, hi = lane >> 5, ql = lane & 31, rep = H / G;
   const int s = tile_seq[tile], t0 = tile_t0[tile], tend = d.seq_off[s + 1], slot = d.slots[s];
   const int tq = HEADS ? t0 : min(t0 + ql, tend - 1);
-  const int g = HEADS ? blockIdx.y * rep + min(ql, rep - 1) : blockIdx.y;
+  const int g = HEADS ? blockIdx.y * rep + min(ql, rep - 1) : blockIdx.y * NW + wv;
   const bool valid_q = HEADS ? ql < rep : t0 + ql < tend;
   const int pos_q = d.tok_pos[tq], pmax = HEADS ? pos_q : d.tok_pos[min(t0 + 31, tend - 1)];
-  const int nds = dk >> 4, ndt = dv >> 5, LD = dv + 8, GV = G * dv, kh = HEADS ? blockIdx.y : g / rep;
+  const int nds = dk >> 4, ndt = dv >> 5, LD = dv + 8, LDK = dk + 8, GV = G * dv, kh = HEADS ? blockIdx.y : g / rep;
   const float sl2 = scale * 1.4426950408889634f;   // scores in units of log2: v_exp_f32 is 2^x
+  const int trow = 4 * (lane >> 5) + ((lane & 15) >> 2), tcol = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
   const int per = (pmax + nsplit) / nsplit, j0 = z * per, j1 = min(pmax + 1, j0 + per);
   const bf16* kbase = kc + ((size_t)slot * max_len) * (G * dk) + kh * dk + 8 * hi;
   const bf16* vbase = vc + ((size_t)slot * max_len) * GV + c * dv;
@@ -116,18 +126,26 @@ __global__ __launch_bounds__(64) void k_talk_attn_mfma(const bf16* __restrict__ 
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[dt][r] = 0.f;
   float m = -INFINITY, l = 0.f;
-  const int vpr = dv >> 3;                       // 16 B vectors per value row
+  const int vpr = dv >> 3, kpr = dk >> 3;        // 16 B vectors per value / key row
   for (int jb = j0; jb < j1; jb += 32) {
     __syncthreads();
-    for (int e = lane; e < 32 * vpr; e += 64) {
+    for (int e = threadIdx.x; e < 32 * vpr; e += 64 * NW) {
       const int row = e / vpr, cv = e % vpr;
       *reinterpret_cast<bf16x8*>(sV + row * LD + cv * 8) =
           *reinterpret_cast<const bf16x8*>(vbase + (size_t)min(jb + row, max_len - 1) * GV + cv * 8);
     }
+    if (NW > 1) {
+      for (int e = threadIdx.x; e < 32 * kpr; e += 64 * NW) {
+        const int row = e / kpr, cv = e % kpr;
+        *reinterpret_cast<bf16x8*>(sK + row * LDK + cv * 8) =
+            *reinterpret_cast<const bf16x8*>(kbase - 8 * hi + (size_t)min(jb + row, max_len - 1) * (G * dk) + cv * 8);
+      }
+      __syncthreads();
+    }
     f32x16 sc;
 #pragma unroll
     for (int r = 0; r < 16; ++r) sc[r] = 0.f;
-    const bf16* kr = kbase + (size_t)min(jb + ql, max_len - 1) * (G * dk);
+    const bf16* kr = NW > 1 ? sK + ql * LDK + 8 * hi : kbase + (size_t)min(jb + ql, max_len - 1) * (G * dk);
 #pragma unroll
     for (int ds = 0; ds < NDS; ++ds)
       if (ds < nds)
@@ -155,7 +173,7 @@ __global__ __launch_bounds__(64) void k_talk_attn_mfma(const bf16* __restrict__ 
     for (int dt = 0; dt < NDT; ++dt)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[dt][r] *= corr;
-    __syncthreads();
+    if (NW == 1) __syncthreads();                  // (four waves: the barrier after the tile copies covers V too)
 #pragma unroll
     for (int u2 = 0; u2 < 2; ++u2) {
       bf16x8 pb;
@@ -164,12 +182,11 @@ __global__ __launch_bounds__(64) void k_talk_attn_mfma(const bf16* __restrict__ 
 #pragma unroll
       for (int dt = 0; dt < NDT; ++dt)
         if (dt < ndt) {
-          bf16x8 vf;
-#pragma unroll
-          for (int j = 0; j < 8; ++j) {
-            const int r = 8 * u2 + j;
-            vf[j] = sV[((r & 3) + 8 * (r >> 2) + 4 * hi) * LD + dt * 32 + ql];
-          }
+          // transposing LDS reads: the 16 lanes of a group address a 4-key x 16-column block (lane 4q'+p': key q',
+          // columns 4p'..4p'+3) and lane i receives column i's four keys; keys 16u2 + 4hi + 0..3, then the same + 8
+          const bf16* vp = sV + (16 * u2 + trow) * LD + dt * 32 + tcol;
+          const bf16x4 v0 = tr_read(vp), v1 = tr_read(vp + 8 * LD);
+          const bf16x8 vf = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
           acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pb, acc[dt], 0, 0, 0);
         }
     }
@@ -245,14 +262,16 @@ void seq_talk_attention(int code, const void* q, int ldq, const void* kc, const 
   if (d.Ttot == 0) return;
   if (tile_seq != nullptr && seq_attn_mfma_ok(code, ldq, dk, dv)) {
     const bool heads = ntiles == d.Ttot && H / G <= 32 && H / G > 1;    // one token per tile: group the heads instead
-    const dim3 grid(ntiles, heads ? G : H, G * nsplit);
-#define SEQ_ATTN_LAUNCH(NDS, NDT, HEADS)                                                                              \
-  hipLaunchKernelGGL((k_talk_attn_mfma<NDS, NDT, HEADS>), grid, dim3(64), 0, st, (const bf16*)q, ldq, (const bf16*)kc, \
-                     (const bf16*)vc, pm, pl, pu, tile_seq, tile_t0, H, G, dk, dv, max_len, nsplit, scale, d)
+    const int nw = (!heads && (H / G) % 4 == 0) ? 4 : 1;                 // four heads of a kv head share its tiles
+    const dim3 grid(ntiles, heads ? G : H / nw, G * nsplit);
+#define SEQ_ATTN_LAUNCH(NDS, NDT, HEADS, NW)                                                                        \
+  hipLaunchKernelGGL((k_talk_attn_mfma<NDS, NDT, HEADS, NW>), grid, dim3(64 * NW), 0, st, (const bf16*)q, ldq,       \
+                     (const bf16*)kc, (const bf16*)vc, pm, pl, pu, tile_seq, tile_t0, H, G, dk, dv, max_len, nsplit, \
+                     scale, d)
     if (dk <= 128 && dv <= 128) {
-      if (heads) SEQ_ATTN_LAUNCH(8, 4, true); else SEQ_ATTN_LAUNCH(8, 4, false);
+      if (heads) SEQ_ATTN_LAUNCH(8, 4, true, 1); else if (nw == 4) SEQ_ATTN_LAUNCH(8, 4, false, 4); else SEQ_ATTN_LAUNCH(8, 4, false, 1);
     } else {
-      if (heads) SEQ_ATTN_LAUNCH(16, 8, true); else SEQ_ATTN_LAUNCH(16, 8, false);
+      if (heads) SEQ_ATTN_LAUNCH(16, 8, true, 1); else if (nw == 4) SEQ_ATTN_LAUNCH(16, 8, false, 4); else SEQ_ATTN_LAUNCH(16, 8, false, 1);
     }
 #undef SEQ_ATTN_LAUNCH
     launch_merge<bf16>(pm, pl, pu, talk, (const bf16*)gate, ldg, (bf16*)out, d.Ttot, H, G, dv, nsplit, st);

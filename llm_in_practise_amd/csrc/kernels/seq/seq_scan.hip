@@ -149,14 +149,41 @@ __device__ __forceinline__ void store_rows(float* p, int r0, int dk, const float
   }
 }
 
-// stage n tokens of a [*, ld] matrix's dk columns at `col0` into LDS rows of DKP floats (zero / `pad` past dk)
-template <typename T, int DKP>
-__device__ __forceinline__ void stage_rows(float* dst, const T* __restrict__ src, size_t ld, int col0, int dk, int n,
+// Staging of a chunk of CT tokens goes through registers: fetch_rows issues all of a lane's loads back to back (one
+// latency, and the next chunk's loads fly while the current chunk is computed), commit_rows writes them to LDS rows
+// of DKP = 16 R floats (`pad` past dk).  CT * DKP / 256 = R elements per lane.
+template <typename T, int R>
+__device__ __forceinline__ void fetch_rows(float (&v)[R], const T* __restrict__ src, size_t ld, int col0, int dk, int n,
                                            float mul, float pad) {
-  for (int e = threadIdx.x; e < n * DKP; e += 256) {
-    const int tt = e / DKP, r = e % DKP;
-    dst[e] = r < dk ? (float)src[(size_t)tt * ld + col0 + r] * mul : pad;
+  constexpr int DKP = KR * R;
+#pragma unroll
+  for (int i = 0; i < R; ++i) {
+    const int e = threadIdx.x + 256 * i, tt = e / DKP, r = e % DKP;
+    v[i] = (tt < n && r < dk) ? (float)src[(size_t)tt * ld + col0 + r] * mul : pad;
   }
+}
+template <int R>
+__device__ __forceinline__ void commit_rows(float* dst, const float (&v)[R]) {
+#pragma unroll
+  for (int i = 0; i < R; ++i) dst[threadIdx.x + 256 * i] = v[i];
+}
+// the chunk's value columns of this block: CT * NC / 256 = 16 / R elements per lane (at least one)
+template <typename T, int R>
+__device__ __forceinline__ void fetch_cols(float (&v)[(16 + R - 1) / R], const T* __restrict__ src, size_t ld, int col0,
+                                           int cb, int dv, int n) {
+  constexpr int NC = 256 / R, PER = (16 + R - 1) / R;
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    const int e = threadIdx.x + 256 * i, tt = e / NC, cc = cb * NC + e % NC;
+    v[i] = (e < CT * NC && tt < n && cc < dv) ? (float)src[(size_t)tt * ld + col0 + cc] : 0.f;
+  }
+}
+template <int R>
+__device__ __forceinline__ void commit_cols(float* dst, const float (&v)[(16 + R - 1) / R]) {
+  constexpr int NC = 256 / R, PER = (16 + R - 1) / R;
+#pragma unroll
+  for (int i = 0; i < PER; ++i)
+    if (threadIdx.x + 256 * i < CT * NC) dst[threadIdx.x + 256 * i] = v[i];
 }
 
 // mLSTM.  m_t = max(f + m, i); S = e^(f+m-m_t) S + e^(i-m_t) k v^T; n likewise; o = S^T q / (max(|n.q|, e^-m_t) + 1e-6)
@@ -172,7 +199,7 @@ __global__ __launch_bounds__(256) void k_mlstm_scan(const T* __restrict__ q, int
   __shared__ __attribute__((aligned(16))) float sk[CT * DKP];
   __shared__ __attribute__((aligned(16))) float sq[CT * DKP];
   __shared__ float sv[CT * NC];
-  __shared__ float sg[2 * CT];
+  __shared__ float sg[4 * CT];
   const int s = blockIdx.x / H, hd = blockIdx.x % H, cb = blockIdx.y, tid = threadIdx.x;
   if (d.live && !d.live[s]) return;
   const int rg = tid % R, cl = tid / R, col = cb * NC + cl, r0 = rg * KR;
@@ -184,26 +211,55 @@ __global__ __launch_bounds__(256) void k_mlstm_scan(const T* __restrict__ q, int
   float m = p0 > 0 ? M[hbase] : 0.f;
   load_rows(Sp, r0, dk, p0 > 0 && colok, Sr);
   load_rows(N + hbase * dk, r0, dk, p0 > 0, nr);
+  float fk[R], fq[R], fv[(16 + R - 1) / R], fi = 0.f, ff = 0.f;
+  auto fetch = [&](int c0) {
+    const int n = min(CT, t1 - c0);
+    fetch_rows<T, R>(fk, k + (size_t)c0 * ldk, ldk, hd * dk, dk, n, 1.f, 0.f);
+    fetch_rows<T, R>(fq, q + (size_t)c0 * ldq, ldq, hd * dk, dk, n, qscale, 0.f);
+    fetch_cols<T, R>(fv, v + (size_t)c0 * ldv, ldv, hd * dv, cb, dv, n);
+    if (tid < n) {
+      fi = ipre[(size_t)(c0 + tid) * H + hd];
+      ff = fpre[(size_t)(c0 + tid) * H + hd];
+    }
+  };
+  if (t0 < t1) fetch(t0);
   for (int c0 = t0; c0 < t1; c0 += CT) {
     const int n = min(CT, t1 - c0);
     __syncthreads();
-    stage_rows<T, DKP>(sk, k + (size_t)c0 * ldk, ldk, hd * dk, dk, n, 1.f, 0.f);
-    stage_rows<T, DKP>(sq, q + (size_t)c0 * ldq, ldq, hd * dk, dk, n, qscale, 0.f);
-    for (int e = tid; e < n * NC; e += 256) {
-      const int tt = e / NC, cc = cb * NC + e % NC;
-      sv[e] = cc < dv ? (float)v[(size_t)(c0 + tt) * ldv + hd * dv + cc] : 0.f;
-    }
-    if (tid < n) {
-      const float ip = ipre[(size_t)(c0 + tid) * H + hd] + ib[hd], fp = fpre[(size_t)(c0 + tid) * H + hd] + fb[hd];
-      sg[2 * tid] = cap * tanhf(ip / cap);
-      sg[2 * tid + 1] = logsigmoidf_(cap * tanhf(fp / cap));
+    commit_rows<R>(sk, fk);
+    commit_rows<R>(sq, fq);
+    commit_cols<R>(sv, fv);
+    if (tid < CT) {
+      // the running maximum is a (max, +) recurrence of the gates alone: with F_t the prefix sum of the log forget
+      // gates, m_t = F_t + max(m_0, max_{s<=t}(i_s - F_s)).  Lanes 0..15 solve the chunk's 16 steps with two
+      // 4-step prefix scans and hand every token its decay e^(f+m'-m), input weight e^(i-m) and floor e^(-m).
+      const bool on = tid < n;
+      const float ig = on ? cap * tanhf((fi + ib[hd]) / cap) : -INFINITY;
+      const float fg = on ? logsigmoidf_(cap * tanhf((ff + fb[hd]) / cap)) : 0.f;
+      float F = fg;
+#pragma unroll
+      for (int o = 1; o < CT; o <<= 1) {
+        const float t = __shfl_up(F, o, CT);
+        if (tid >= o) F += t;
+      }
+      float pm = ig - F;
+#pragma unroll
+      for (int o = 1; o < CT; o <<= 1) {
+        const float t = __shfl_up(pm, o, CT);
+        if (tid >= o) pm = fmaxf(pm, t);
+      }
+      const float mt = F + fmaxf(m, pm);
+      float mp = __shfl_up(mt, 1, CT);
+      if (tid == 0) mp = m;
+      sg[4 * tid] = expf(fg + mp - mt);
+      sg[4 * tid + 1] = expf(ig - mt);
+      sg[4 * tid + 2] = expf(-mt);
+      sg[4 * tid + 3] = mt;
     }
     __syncthreads();
+    if (c0 + CT < t1) fetch(c0 + CT);
     for (int tt = 0; tt < n; ++tt) {
-      const float ig = sg[2 * tt], fg = sg[2 * tt + 1];
-      const float mn = fmaxf(fg + m, ig);
-      const float a = expf(fg + m - mn), b = expf(ig - mn);
-      m = mn;
+      const float a = sg[4 * tt], b = sg[4 * tt + 1];
       const float bv = b * sv[tt * NC + cl];
       float num[4] = {0.f, 0.f, 0.f, 0.f}, den[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -222,8 +278,9 @@ __global__ __launch_bounds__(256) void k_mlstm_scan(const T* __restrict__ q, int
       const float nm = group_sum<R>((num[0] + num[1]) + (num[2] + num[3]));
       const float dn = group_sum<R>((den[0] + den[1]) + (den[2] + den[3]));
       if (rg == 0 && colok)
-        out[((size_t)(c0 + tt) * H + hd) * dv + col] = nm / (fmaxf(fabsf(dn), expf(-m)) + 1e-6f);
+        out[((size_t)(c0 + tt) * H + hd) * dv + col] = nm / (fmaxf(fabsf(dn), sg[4 * tt + 2]) + 1e-6f);
     }
+    m = sg[4 * (n - 1) + 3];
   }
   if (colok) store_rows(Sp, r0, dk, Sr);
   if (cb == 0 && cl == 0) store_rows(N + hbase * dk, r0, dk, nr);
@@ -251,18 +308,26 @@ __global__ __launch_bounds__(256) void k_delta_scan(const T* __restrict__ q, int
   float* Sp = S + (((size_t)slot * H + hd) * dv + (colok ? col : 0)) * dk;
   float Sr[KR];
   load_rows(Sp, r0, dk, p0 > 0 && colok, Sr);
+  float fk[R], fq[R], fd[R], fv[(16 + R - 1) / R], fb = 0.f;
+  auto fetch = [&](int c0) {
+    const int n = min(CT, t1 - c0);
+    fetch_rows<T, R>(fk, k + (size_t)c0 * ldk, ldk, kh * dk, dk, n, 1.f, 0.f);
+    fetch_rows<T, R>(fq, q + (size_t)c0 * ldq, ldq, kh * dk, dk, n, 1.f, 0.f);
+    fetch_rows<float, R>(fd, g + (size_t)c0 * H * dk, (size_t)H * dk, hd * dk, dk, n, 1.f, 1.f);
+    fetch_cols<T, R>(fv, v + (size_t)c0 * ldv, ldv, hd * dv, cb, dv, n);
+    if (tid < n) fb = bpre[(size_t)(c0 + tid) * H + hd];
+  };
+  if (t0 < t1) fetch(t0);
   for (int c0 = t0; c0 < t1; c0 += CT) {
     const int n = min(CT, t1 - c0);
     __syncthreads();
-    stage_rows<T, DKP>(sk, k + (size_t)c0 * ldk, ldk, kh * dk, dk, n, 1.f, 0.f);
-    stage_rows<T, DKP>(sq, q + (size_t)c0 * ldq, ldq, kh * dk, dk, n, 1.f, 0.f);
-    stage_rows<float, DKP>(sd, g + (size_t)c0 * H * dk, (size_t)H * dk, hd * dk, dk, n, 1.f, 1.f);
-    for (int e = tid; e < n * NC; e += 256) {
-      const int tt = e / NC, cc = cb * NC + e % NC;
-      sv[e] = cc < dv ? (float)v[(size_t)(c0 + tt) * ldv + hd * dv + cc] : 0.f;
-    }
-    if (tid < n) sb[tid] = sigmoidf_(bpre[(size_t)(c0 + tid) * H + hd]);
+    commit_rows<R>(sk, fk);
+    commit_rows<R>(sq, fq);
+    commit_rows<R>(sd, fd);
+    commit_cols<R>(sv, fv);
+    if (tid < n) sb[tid] = sigmoidf_(fb);
     __syncthreads();
+    if (c0 + CT < t1) fetch(c0 + CT);
     for (int tt = 0; tt < n; ++tt) {
       f32x4 kk[KR / 4];
       float dot[4] = {0.f, 0.f, 0.f, 0.f};

@@ -403,7 +403,8 @@ def test_decode_graphs_replay_equals_eager():
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("dk,dv,H,G", [(32, 32, 4, 2), (64, 128, 6, 3), (144, 160, 2, 1), (128, 64, 8, 8)])
+@pytest.mark.parametrize("dk,dv,H,G", [(32, 32, 4, 2), (64, 128, 6, 3), (144, 160, 2, 1), (128, 64, 8, 8), (64, 64, 8, 2),
+                                       (160, 192, 4, 1), (16, 32, 16, 2)])
 @pytest.mark.parametrize("scale", [0.2, 4.0])
 def test_matrix_core_attention_sweep(dk, dv, H, G, scale):
     """bf16 head-mixing attention on the matrix-core kernel (ragged batch, continued sequences, tiles that end inside
@@ -443,7 +444,8 @@ def test_matrix_core_attention_sweep(dk, dv, H, G, scale):
 @pytest.mark.parametrize("device", DEVICES)
 def test_bf16_matrix_core_sizes_long_context(device):
     """bf16 model whose attention sizes take the matrix-core path; 600 tokens, then decoding across key splits."""
-    cfg = config([parallel(lh=4, lg=2, ldim=32, lvdim=32, lconv=3, scale=0.25, mlp=None), mlstm()], width=64)
+    cfg = config([parallel(lh=8, lg=2, ldim=32, lvdim=32, lconv=3, scale=0.25, mlp=None),
+                  parallel(lh=4, lg=2, ldim=64, lvdim=32, lconv=2, scale=0.125, mlp=32)], width=64)
     lm, W = build(cfg, device, seed=12, dtype=torch.bfloat16)
     toks = tokens(620, cfg["vocab"], 19)
     got = replay(lm, 1100, [([("a", toks[:600])], [])] + [([("a", [t])], []) for t in toks[600:]])["a"]
