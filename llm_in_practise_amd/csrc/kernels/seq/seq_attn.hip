@@ -127,20 +127,45 @@ __global__ __launch_bounds__(64 * NW) void k_talk_attn_mfma(const bf16* __restri
     for (int r = 0; r < 16; ++r) acc[dt][r] = 0.f;
   float m = -INFINITY, l = 0.f;
   const int vpr = dv >> 3, kpr = dk >> 3;        // 16 B vectors per value / key row
+  // four waves: the next key / value tile is fetched into registers while the current one is computed on
+  constexpr int VPT = NW > 1 ? (2 * NDT) / NW : 1, KPT = NW > 1 ? (2 * NDS) / NW : 1;
+  bf16x8 pv[VPT], pk[KPT];
+  auto fetch = [&](int jb) {
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+      const int e = threadIdx.x + 64 * NW * i, row = e / vpr, cv = e % vpr;
+      if (e < 32 * vpr)
+        pv[i] = *reinterpret_cast<const bf16x8*>(vbase + (size_t)min(jb + row, max_len - 1) * GV + cv * 8);
+    }
+#pragma unroll
+    for (int i = 0; i < KPT; ++i) {
+      const int e = threadIdx.x + 64 * NW * i, row = e / kpr, cv = e % kpr;
+      if (e < 32 * kpr)
+        pk[i] = *reinterpret_cast<const bf16x8*>(kbase - 8 * hi + (size_t)min(jb + row, max_len - 1) * (G * dk) + cv * 8);
+    }
+  };
+  if (NW > 1 && j0 < j1) fetch(j0);
   for (int jb = j0; jb < j1; jb += 32) {
     __syncthreads();
-    for (int e = threadIdx.x; e < 32 * vpr; e += 64 * NW) {
-      const int row = e / vpr, cv = e % vpr;
-      *reinterpret_cast<bf16x8*>(sV + row * LD + cv * 8) =
-          *reinterpret_cast<const bf16x8*>(vbase + (size_t)min(jb + row, max_len - 1) * GV + cv * 8);
-    }
     if (NW > 1) {
-      for (int e = threadIdx.x; e < 32 * kpr; e += 64 * NW) {
-        const int row = e / kpr, cv = e % kpr;
-        *reinterpret_cast<bf16x8*>(sK + row * LDK + cv * 8) =
-            *reinterpret_cast<const bf16x8*>(kbase - 8 * hi + (size_t)min(jb + row, max_len - 1) * (G * dk) + cv * 8);
+#pragma unroll
+      for (int i = 0; i < VPT; ++i) {
+        const int e = threadIdx.x + 64 * NW * i;
+        if (e < 32 * vpr) *reinterpret_cast<bf16x8*>(sV + (e / vpr) * LD + (e % vpr) * 8) = pv[i];
+      }
+#pragma unroll
+      for (int i = 0; i < KPT; ++i) {
+        const int e = threadIdx.x + 64 * NW * i;
+        if (e < 32 * kpr) *reinterpret_cast<bf16x8*>(sK + (e / kpr) * LDK + (e % kpr) * 8) = pk[i];
       }
       __syncthreads();
+      if (jb + 32 < j1) fetch(jb + 32);
+    } else {
+      for (int e = threadIdx.x; e < 32 * vpr; e += 64) {
+        const int row = e / vpr, cv = e % vpr;
+        *reinterpret_cast<bf16x8*>(sV + row * LD + cv * 8) =
+            *reinterpret_cast<const bf16x8*>(vbase + (size_t)min(jb + row, max_len - 1) * GV + cv * 8);
+      }
     }
     f32x16 sc;
 #pragma unroll
