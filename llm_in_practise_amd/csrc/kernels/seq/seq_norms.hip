@@ -100,18 +100,24 @@ __global__ __launch_bounds__(256) void k_polynorm(const T* __restrict__ z, const
   }
 }
 
-// out[t, h, c] = o[t, h, c] / rms_c(o[t, h, :]) * w[(per_head ? h * dv : 0) + c] * sigmoid(gate[t, h * dv + c])
+// out[t, h, c] = o[t, h, c] / rms_c(o[t, h, :]) * w[(per_head ? h * dv : 0) + c] * sigmoid(gate[t, h * dv + c]);
+// with den / efl (per token and head) o is first divided by max(|den|, efl) + 1e-6 (the mLSTM read-out)
 template <typename T>
 __global__ __launch_bounds__(256) void k_head_norm_gate(const float* __restrict__ o, const float* __restrict__ w,
                                                         int per_head, const T* __restrict__ gate, int ldg,
+                                                        const float* __restrict__ den, const float* __restrict__ efl,
                                                         T* __restrict__ out, int nrows, int H, int dv, float eps) {
   const int row = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
   if (row >= nrows) return;
   const int t = row / H, hd = row % H;
   const float* src = o + (size_t)row * dv;
+  const float dinv = den != nullptr ? 1.f / (fmaxf(fabsf(den[row]), efl[row]) + 1e-6f) : 1.f;
   float s = 0.f;
-  for (int c = lane; c < dv; c += 64) s += src[c] * src[c];
-  const float rs = rsqrtf(wave_sum(s) / dv + eps);
+  for (int c = lane; c < dv; c += 64) {
+    const float v = src[c] * dinv;
+    s += v * v;
+  }
+  const float rs = rsqrtf(wave_sum(s) / dv + eps) * dinv;
   for (int c = lane; c < dv; c += 64) {
     const float g = sigmoidf_((float)gate[(size_t)t * ldg + hd * dv + c]);
     out[(size_t)row * dv + c] = (T)(src[c] * rs * w[(per_head ? hd * dv : 0) + c] * g);
@@ -166,12 +172,12 @@ void seq_polynorm(int code, const void* z, const float* coef, void* out, int T_,
   LIPA_CHECK_LAUNCH();
 }
 
-void seq_head_norm_gate(int code, const float* o, const float* w, int per_head, const void* gate, int ldg, void* out,
-                        int T_, int H, int dv, float eps, hipStream_t st) {
+void seq_head_norm_gate(int code, const float* o, const float* w, int per_head, const void* gate, int ldg,
+                        const float* den, const float* efl, void* out, int T_, int H, int dv, float eps, hipStream_t st) {
   const int rows = T_ * H;
   if (rows == 0) return;
   SEQ_DISPATCH_T(code, hipLaunchKernelGGL(k_head_norm_gate<T>, dim3((rows + 3) / 4), dim3(256), 0, st, o, w, per_head,
-                                          (const T*)gate, ldg, (T*)out, rows, H, dv, eps));
+                                          (const T*)gate, ldg, den, efl, (T*)out, rows, H, dv, eps));
   LIPA_CHECK_LAUNCH();
 }
 

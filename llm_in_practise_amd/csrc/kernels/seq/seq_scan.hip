@@ -168,14 +168,15 @@ __device__ __forceinline__ void commit_rows(float* dst, const float (&v)[R]) {
   for (int i = 0; i < R; ++i) dst[threadIdx.x + 256 * i] = v[i];
 }
 // the chunk's value columns of this block: CT * NC / 256 = 16 / R elements per lane (at least one)
+// (ones: column dv reads as 1 — the mLSTM's normaliser vector is the state column whose value is always 1)
 template <typename T, int R>
 __device__ __forceinline__ void fetch_cols(float (&v)[(16 + R - 1) / R], const T* __restrict__ src, size_t ld, int col0,
-                                           int cb, int dv, int n) {
+                                           int cb, int dv, int n, bool ones = false) {
   constexpr int NC = 256 / R, PER = (16 + R - 1) / R;
 #pragma unroll
   for (int i = 0; i < PER; ++i) {
     const int e = threadIdx.x + 256 * i, tt = e / NC, cc = cb * NC + e % NC;
-    v[i] = (e < CT * NC && tt < n && cc < dv) ? (float)src[(size_t)tt * ld + col0 + cc] : 0.f;
+    v[i] = (e < CT * NC && tt < n && cc < dv) ? (float)src[(size_t)tt * ld + col0 + cc] : (ones && cc == dv ? 1.f : 0.f);
   }
 }
 template <int R>
@@ -188,13 +189,16 @@ __device__ __forceinline__ void commit_cols(float* dst, const float (&v)[(16 + R
 
 // mLSTM.  m_t = max(f + m, i); S = e^(f+m-m_t) S + e^(i-m_t) k v^T; n likewise; o = S^T q / (max(|n.q|, e^-m_t) + 1e-6)
 // with i = cap tanh((ipre + ib) / cap), f = logsigmoid(cap tanh((fpre + fb) / cap)); m starts at 0.
+// The normaliser n obeys S's recurrence with v = 1, so it runs as column dv of the same scan; the kernel writes the
+// numerators S^T q, and per (token, head) the normaliser product n.q and the floor e^-m; the read-out kernel divides.
 template <typename T, int R>
 __global__ __launch_bounds__(256) void k_mlstm_scan(const T* __restrict__ q, int ldq, const T* __restrict__ k, int ldk,
                                                     const T* __restrict__ v, int ldv, const float* __restrict__ ipre,
                                                     const float* __restrict__ fpre, const float* __restrict__ ib,
                                                     const float* __restrict__ fb, float cap, float qscale,
                                                     float* __restrict__ S, float* __restrict__ N, float* __restrict__ M,
-                                                    float* __restrict__ out, int H, int dk, int dv, SeqDesc d) {
+                                                    float* __restrict__ out, float* __restrict__ den,
+                                                    float* __restrict__ efl, int H, int dk, int dv, SeqDesc d) {
   constexpr int DKP = KR * R, NC = 256 / R;
   __shared__ __attribute__((aligned(16))) float sk[CT * DKP];
   __shared__ __attribute__((aligned(16))) float sq[CT * DKP];
@@ -203,20 +207,19 @@ __global__ __launch_bounds__(256) void k_mlstm_scan(const T* __restrict__ q, int
   const int s = blockIdx.x / H, hd = blockIdx.x % H, cb = blockIdx.y, tid = threadIdx.x;
   if (d.live && !d.live[s]) return;
   const int rg = tid % R, cl = tid / R, col = cb * NC + cl, r0 = rg * KR;
-  const bool colok = col < dv;
+  const bool colok = col <= dv, isn = col == dv;          // column dv is the normaliser
   const int t0 = d.seq_off[s], t1 = d.seq_off[s + 1], p0 = d.pos0[s], slot = d.slots[s];
   const size_t hbase = (size_t)slot * H + hd;
-  float* Sp = S + (hbase * dv + (colok ? col : 0)) * dk;
-  float Sr[KR], nr[KR];
+  float* Sp = isn ? N + hbase * dk : S + (hbase * dv + (colok ? col : 0)) * dk;
+  float Sr[KR];
   float m = p0 > 0 ? M[hbase] : 0.f;
   load_rows(Sp, r0, dk, p0 > 0 && colok, Sr);
-  load_rows(N + hbase * dk, r0, dk, p0 > 0, nr);
   float fk[R], fq[R], fv[(16 + R - 1) / R], fi = 0.f, ff = 0.f;
   auto fetch = [&](int c0) {
     const int n = min(CT, t1 - c0);
     fetch_rows<T, R>(fk, k + (size_t)c0 * ldk, ldk, hd * dk, dk, n, 1.f, 0.f);
     fetch_rows<T, R>(fq, q + (size_t)c0 * ldq, ldq, hd * dk, dk, n, qscale, 0.f);
-    fetch_cols<T, R>(fv, v + (size_t)c0 * ldv, ldv, hd * dv, cb, dv, n);
+    fetch_cols<T, R>(fv, v + (size_t)c0 * ldv, ldv, hd * dv, cb, dv, n, true);
     if (tid < n) {
       fi = ipre[(size_t)(c0 + tid) * H + hd];
       ff = fpre[(size_t)(c0 + tid) * H + hd];
@@ -255,13 +258,14 @@ __global__ __launch_bounds__(256) void k_mlstm_scan(const T* __restrict__ q, int
       sg[4 * tid + 1] = expf(ig - mt);
       sg[4 * tid + 2] = expf(-mt);
       sg[4 * tid + 3] = mt;
+      if (on && cb == 0) efl[(size_t)(c0 + tid) * H + hd] = expf(-mt);
     }
     __syncthreads();
     if (c0 + CT < t1) fetch(c0 + CT);
     for (int tt = 0; tt < n; ++tt) {
       const float a = sg[4 * tt], b = sg[4 * tt + 1];
       const float bv = b * sv[tt * NC + cl];
-      float num[4] = {0.f, 0.f, 0.f, 0.f}, den[4] = {0.f, 0.f, 0.f, 0.f};
+      float num[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int i4 = 0; i4 < KR / 4; ++i4) {
         const f32x4 kk = *reinterpret_cast<const f32x4*>(sk + tt * DKP + r0 + 4 * i4);
@@ -270,20 +274,20 @@ __global__ __launch_bounds__(256) void k_mlstm_scan(const T* __restrict__ q, int
         for (int j = 0; j < 4; ++j) {
           const int i = 4 * i4 + j;
           Sr[i] = a * Sr[i] + kk[j] * bv;
-          nr[i] = a * nr[i] + b * kk[j];
           num[j] += Sr[i] * qq[j];
-          den[j] += nr[i] * qq[j];
         }
       }
       const float nm = group_sum<R>((num[0] + num[1]) + (num[2] + num[3]));
-      const float dn = group_sum<R>((den[0] + den[1]) + (den[2] + den[3]));
-      if (rg == 0 && colok)
-        out[((size_t)(c0 + tt) * H + hd) * dv + col] = nm / (fmaxf(fabsf(dn), sg[4 * tt + 2]) + 1e-6f);
+      if (rg == 0 && colok) {
+        if (isn)
+          den[(size_t)(c0 + tt) * H + hd] = nm;
+        else
+          out[((size_t)(c0 + tt) * H + hd) * dv + col] = nm;
+      }
     }
     m = sg[4 * (n - 1) + 3];
   }
   if (colok) store_rows(Sp, r0, dk, Sr);
-  if (cb == 0 && cl == 0) store_rows(N + hbase * dk, r0, dk, nr);
   if (cb == 0 && tid == 0) M[hbase] = m;
 }
 
@@ -407,13 +411,14 @@ void seq_short_conv(int code, int out_f32, const void* u, int ldu, const float* 
 
 void seq_mlstm_scan(int code, const void* q, int ldq, const void* k, int ldk, const void* v, int ldv, const float* ipre,
                     const float* fpre, const float* ib, const float* fb, float cap, float qscale, float* S, float* N,
-                    float* M, float* out, int H, int dk, int dv, SeqDesc d, hipStream_t st) {
+                    float* M, float* out, float* den, float* efl, int H, int dk, int dv, SeqDesc d, hipStream_t st) {
   if (d.B == 0) return;
   const int Rr = rows_split(dk);
   SEQ_DISPATCH_T(code, SEQ_DISPATCH_R(Rr, {
     constexpr int NC = 256 / R;
-    hipLaunchKernelGGL((k_mlstm_scan<T, R>), dim3(d.B * H, (dv + NC - 1) / NC), dim3(256), 0, st, (const T*)q, ldq,
-                       (const T*)k, ldk, (const T*)v, ldv, ipre, fpre, ib, fb, cap, qscale, S, N, M, out, H, dk, dv, d);
+    hipLaunchKernelGGL((k_mlstm_scan<T, R>), dim3(d.B * H, (dv + 1 + NC - 1) / NC), dim3(256), 0, st, (const T*)q, ldq,
+                       (const T*)k, ldk, (const T*)v, ldv, ipre, fpre, ib, fb, cap, qscale, S, N, M, out, den, efl, H,
+                       dk, dv, d);
   }));
   LIPA_CHECK_LAUNCH();
 }

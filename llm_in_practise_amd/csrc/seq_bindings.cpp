@@ -26,13 +26,14 @@ void seq_gated_residual(int, float*, const void*, int, const void*, int, const f
                         void*, int, int, float, hipStream_t);
 void seq_dual_norm_mean(int, const void*, const void*, const float*, const float*, void*, int, int, float, hipStream_t);
 void seq_polynorm(int, const void*, const float*, void*, int, int, float, hipStream_t);
-void seq_head_norm_gate(int, const float*, const float*, int, const void*, int, void*, int, int, int, float,
-                        hipStream_t);
+void seq_head_norm_gate(int, const float*, const float*, int, const void*, int, const float*, const float*, void*, int,
+                        int, int, float, hipStream_t);
 void seq_decay_gate(const float*, const float*, const float*, float*, int, int, int, hipStream_t);
 void seq_short_conv(int, int, const void*, int, const float*, void*, void*, int, int, int, const int*,
                     const float* const*, const float*, SeqDesc, float, hipStream_t);
 void seq_mlstm_scan(int, const void*, int, const void*, int, const void*, int, const float*, const float*, const float*,
-                    const float*, float, float, float*, float*, float*, float*, int, int, int, SeqDesc, hipStream_t);
+                    const float*, float, float, float*, float*, float*, float*, float*, float*, int, int, int, SeqDesc,
+                    hipStream_t);
 void seq_delta_scan(int, const void*, int, const void*, int, const void*, int, const float*, const float*, float*,
                     float*, int, int, int, int, SeqDesc, hipStream_t);
 void seq_talk_attention(int, const void*, int, const void*, const void*, float*, float*, float*, const float*,
@@ -150,7 +151,8 @@ Tensor polynorm(Tensor z, Tensor coef, double eps) {
   return out;
 }
 
-Tensor head_norm_gate(Tensor o, Tensor w, Tensor gate, double eps) {
+// den / efl (optional, float [T, H]): o is divided by max(|den|, efl) + 1e-6 first
+Tensor head_norm_gate(Tensor o, Tensor w, Tensor gate, double eps, optional<Tensor> den, optional<Tensor> efl) {
   f32c(o, "o");
   TORCH_CHECK(o.dim() == 3, "o: [T, H, dv]");
   const int T = (int)o.size(0), H = (int)o.size(1), dv = (int)o.size(2), code = code_of(gate);
@@ -158,7 +160,17 @@ Tensor head_norm_gate(Tensor o, Tensor w, Tensor gate, double eps) {
   TORCH_CHECK(w.numel() == dv || w.numel() == (int64_t)H * dv, "norm weight: [dv] or [H * dv]");
   rows(gate, T, (int64_t)H * dv, code, "gate");
   auto out = at::empty({T, (int64_t)H * dv}, gate.options());
-  seq_head_norm_gate(code, o.data_ptr<float>(), w.data_ptr<float>(), w.numel() != dv, gate.data_ptr(), ld(gate),
+  const float* dp = nullptr;
+  const float* ep = nullptr;
+  if (den && den->defined()) {
+    TORCH_CHECK(efl && efl->defined(), "den comes with efl");
+    f32c(*den, "den");
+    f32c(*efl, "efl");
+    TORCH_CHECK(den->numel() == (int64_t)T * H && efl->numel() == (int64_t)T * H, "den / efl: [T, H]");
+    dp = den->data_ptr<float>();
+    ep = efl->data_ptr<float>();
+  }
+  seq_head_norm_gate(code, o.data_ptr<float>(), w.data_ptr<float>(), w.numel() != dv, gate.data_ptr(), ld(gate), dp, ep,
                      out.data_ptr(), T, H, dv, (float)eps, stream());
   return out;
 }
@@ -228,7 +240,8 @@ static void check_state(const Tensor& S, int64_t H, int64_t dv, int64_t dk) {
   TORCH_CHECK(S.dim() == 4 && S.size(1) == H && S.size(2) == dv && S.size(3) == dk, "state: [slots, H, dv, dk]");
 }
 
-Tensor mlstm_scan(Tensor q, Tensor k, Tensor v, Tensor ipre, Tensor fpre, Tensor ib, Tensor fb, double cap,
+// returns {numerators S^T q [T, H, dv], n.q [T, H], e^-m [T, H]}: the read-out kernel divides
+std::vector<Tensor> mlstm_scan(Tensor q, Tensor k, Tensor v, Tensor ipre, Tensor fpre, Tensor ib, Tensor fb, double cap,
                   double qscale, Tensor S, Tensor N, Tensor M, int64_t H, std::vector<Tensor> desc,
                   optional<Tensor> live) {
   const int code = code_of(q);
@@ -251,11 +264,12 @@ Tensor mlstm_scan(Tensor q, Tensor k, Tensor v, Tensor ipre, Tensor fpre, Tensor
   TORCH_CHECK(N.numel() == S.size(0) * H * dk && M.numel() == S.size(0) * H, "n / m state sizes");
   SeqDesc d = desc_of(desc, live, T);
   auto out = at::empty({T, H, dv}, S.options());
+  auto den = at::empty({T, H}, S.options()), efl = at::empty({T, H}, S.options());
   seq_mlstm_scan(code, q.data_ptr(), ld(q), k.data_ptr(), ld(k), v.data_ptr(), ld(v), ipre.data_ptr<float>(),
                  fpre.data_ptr<float>(), ib.data_ptr<float>(), fb.data_ptr<float>(), (float)cap, (float)qscale,
-                 S.data_ptr<float>(), N.data_ptr<float>(), M.data_ptr<float>(), out.data_ptr<float>(), (int)H, (int)dk,
-                 (int)dv, d, stream());
-  return out;
+                 S.data_ptr<float>(), N.data_ptr<float>(), M.data_ptr<float>(), out.data_ptr<float>(),
+                 den.data_ptr<float>(), efl.data_ptr<float>(), (int)H, (int)dk, (int)dv, d, stream());
+  return {out, den, efl};
 }
 
 Tensor delta_scan(Tensor q, Tensor k, Tensor v, Tensor g, Tensor bpre, Tensor S, int64_t H, int64_t G,

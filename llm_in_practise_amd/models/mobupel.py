@@ -185,9 +185,10 @@ class MlstmMixer(_Sublayer):
         P = h @ self.w_in.t()
         gates = h.float() @ self.w_gate.t()
         a, b = H * dk, 2 * H * dk
-        o = mlstm_scan(P[:, :a], P[:, a:b], P[:, b:b + H * dv], gates[:, :H].contiguous(), gates[:, H:].contiguous(),
-                       self.ib, self.fb, self.cap, dk ** -0.5, st["S"], st["n"], st["m"], H, sb)
-        y = head_norm_gate(o, self.norm, P[:, b + H * dv:b + 2 * H * dv], eps)
+        o, den, floor = mlstm_scan(P[:, :a], P[:, a:b], P[:, b:b + H * dv], gates[:, :H].contiguous(),
+                                   gates[:, H:].contiguous(), self.ib, self.fb, self.cap, dk ** -0.5, st["S"], st["n"],
+                                   st["m"], H, sb)
+        y = head_norm_gate(o, self.norm, P[:, b + H * dv:b + 2 * H * dv], eps, den, floor)
         return y @ self.w_o.t(), P[:, self.n_in:]
 
 

@@ -143,11 +143,15 @@ def dual_norm_mean(a: torch.Tensor, b: torch.Tensor, wa: torch.Tensor, wb: torch
     return ref.dual_norm_mean(a, b, wa, wb, eps)
 
 
-def head_norm_gate(o: torch.Tensor, weight: torch.Tensor, gate_pre: torch.Tensor, eps: float) -> torch.Tensor:
+def head_norm_gate(o: torch.Tensor, weight: torch.Tensor, gate_pre: torch.Tensor, eps: float,
+                   den: torch.Tensor | None = None, floor: torch.Tensor | None = None) -> torch.Tensor:
     """Read-out of a recurrent mixer: ``o`` float ``[T, H, dv]`` is RMS-normed per head, scaled by ``weight``
     (``[dv]`` shared by the heads or ``[H * dv]``) and multiplied by ``sigmoid(gate_pre)``; returns ``[T, H * dv]``
-    in ``gate_pre``'s dtype."""
+    in ``gate_pre``'s dtype.  With ``den`` / ``floor`` (float ``[T, H]``) ``o`` is first divided by
+    ``max(|den|, floor) + 1e-6`` (the mLSTM's normaliser)."""
     from ._native import native_seq, use_seq
     if use_seq(o):
-        return native_seq().head_norm_gate(o, weight, gate_pre, eps)
+        return native_seq().head_norm_gate(o, weight, gate_pre, eps, den, floor)
+    if den is not None:
+        o = o / (torch.maximum(den.abs(), floor) + 1e-6)[..., None]
     return ref.head_norm_gate(o, weight, gate_pre, eps)

@@ -19,11 +19,14 @@ from ._native import native_seq, use_seq
 def mlstm_scan(q, k, v, i_pre, f_pre, i_bias, f_bias, cap: float, q_scale: float, S, N, M, heads: int, sb):
     """``q, k`` ``[T, H*dk]``, ``v`` ``[T, H*dv]`` (activation dtype), gate pre-activations float ``[T, H]``.
     Gates: ``i = cap*tanh((i_pre+i_bias)/cap)``, ``f = logsigmoid(cap*tanh((f_pre+f_bias)/cap))``; running maximum
-    ``m`` starts at 0.  Returns float ``[T, H, dv]``: ``S^T q / (max(|n.q|, exp(-m)) + 1e-6)``."""
+    ``m`` starts at 0.  Returns ``(o, den, floor)`` for :func:`~.norm.head_norm_gate`: the read-out is
+    ``o / (max(|den|, floor) + 1e-6)`` with ``o = S^T q`` float ``[T, H, dv]``, ``den = n.q`` and ``floor = exp(-m)``
+    float ``[T, H]`` (the HIP scan leaves the division to the read-out kernel; the CPU path returns the divided ``o``
+    and ``None, None``)."""
     if use_seq(q):
-        return native_seq().mlstm_scan(q, k, v, i_pre, f_pre, i_bias, f_bias, cap, q_scale, S, N, M, heads, sb.desc,
-                                       sb.live)
-    return ref.mlstm_scan(q, k, v, i_pre, f_pre, i_bias, f_bias, cap, q_scale, S, N, M, heads, sb)
+        return tuple(native_seq().mlstm_scan(q, k, v, i_pre, f_pre, i_bias, f_bias, cap, q_scale, S, N, M, heads,
+                                             sb.desc, sb.live))
+    return ref.mlstm_scan(q, k, v, i_pre, f_pre, i_bias, f_bias, cap, q_scale, S, N, M, heads, sb), None, None
 
 
 def decay_gate(pre, bias, a_log, dk: int):
