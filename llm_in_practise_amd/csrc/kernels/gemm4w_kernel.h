@@ -122,7 +122,7 @@ __device__ __forceinline__ void dma_lds(const rsrc_t& rs, uint32_t dst, uint32_t
 }
 
 // s_waitcnt immediate for vmcnt(0) alone (the full drain that register loads issued near LDS-DMAs need: a counted
-// vmcnt(N > 0) is never their guard — scripts/vmcnt_audit.py, tests/test_vmcnt_audit_cpu.py)
+// vmcnt(N > 0) is never their guard)
 constexpr int WAIT_VM0 = 0 | (7 << 4) | (15 << 8) | (0 << 14);
 
 // compile-time unrolled loop: f(std::integral_constant<int, k>) for k in [K, N)
@@ -637,8 +637,8 @@ __global__ __launch_bounds__(NT, 1) void gemm4w_k(const bf16* __restrict__ A, in
     //  NT: K-step 0 of the adapters' extra K (xa·Bᵀ) initialises the accumulators;
     //  BT: the masked input-gradient term Σ_b D_b(ds_b·g_b·A_b) initialises them.
     // Operands come by compiler-visible global loads, drained by vmcnt(0) BEFORE the first LDS-DMA is issued:
-    // no counted wait ever guards a register load beside the DMAs (the round-5 dK/dV race:
-    // profiles/r5/zero3_dkv_race.txt; pinned by tests/test_vmcnt_audit_cpu.py).  The loads hit L2 (xa / g were
+    // no counted wait ever guards a register load beside the DMAs (such a wait once let a dK/dV tile race its own
+    // operand loads).  The loads hit L2 (xa / g were
     // written by the launch before), so the drain costs one L2 latency per workgroup.
     bf16x8 lxe[8], lbe[8], lbe2[8], lxe2[8];
     u32x4 lkeep[2][8], lga[2][8], lgb[2][8];
