@@ -346,8 +346,9 @@ class SeqStateCache:
     does for K/V alone.  ``pos`` (int32, device) is each slot's next position; a slot is recycled by starting its
     next sequence at position 0, which makes every kernel ignore what the slot held.
 
-    ``specs``: per layer a dict ``name -> (shape after the slot axis, "act" | "f32" | "kv")``; ``"kv"`` entries get
-    the ``max_len`` axis, ``"act"`` ones the activation dtype."""
+    ``specs``: per layer a dict ``name -> (shape after the slot axis, "act" | "f32" | "i32" | "kv")``; ``"kv"`` entries
+    get the ``max_len`` axis and, like ``"act"`` ones, the activation dtype; ``"i32"`` entries hold integers (a carried
+    token).  A model may append dicts of its own after the layers' (state that belongs to no layer)."""
 
     def __init__(self, specs: list[dict], batch: int, max_len: int, dtype, device):
         self.specs, self.batch, self.max_len, self.dtype, self.device = specs, batch, max_len, dtype, torch.device(device)
@@ -356,7 +357,7 @@ class SeqStateCache:
             d = {}
             for name, (shape, kind) in spec.items():
                 full = (batch, max_len, *shape) if kind == "kv" else (batch, *shape)
-                d[name] = torch.zeros(full, dtype=torch.float32 if kind == "f32" else dtype, device=device)
+                d[name] = torch.zeros(full, dtype={"f32": torch.float32, "i32": torch.int32}.get(kind, dtype), device=device)
             self.layers.append(d)
         self.pos = torch.zeros(batch, dtype=torch.int32, device=device)
         self.live = torch.ones(batch, dtype=torch.int32, device=device)    # rows whose state a decode step may touch
@@ -369,7 +370,7 @@ class SeqStateCache:
     def slot_bytes(specs: list[dict], max_len: int, dtype) -> int:
         import math
         el = torch.finfo(dtype).bits // 8
-        return sum(math.prod(shape) * (max_len * el if kind == "kv" else el if kind == "act" else 4)
+        return sum(math.prod(shape) * (max_len * el if kind == "kv" else el if kind == "act" else 4)   # f32 / i32: 4
                    for spec in specs for shape, kind in spec.values())
 
     # ---- the views the engine and generate() ask a cache for
@@ -396,3 +397,115 @@ class SeqStateCache:
 
     def get_seq_length(self) -> int:
         return self.len
+
+
+class SeqStateModel(nn.Module):
+    """The trunk of a causal LM whose sequences live in a :class:`SeqStateCache`.  A subclass gives
+    :meth:`state_specs` and :meth:`run` (packed tokens -> final-normed hidden states); this class turns the calls
+    of the serving engine (a :class:`SeqBatch`), of ``generate()`` (right-padded prompts, then one token per row)
+    and a plain forward into ``run`` over the right batch view."""
+
+    dtype: torch.dtype
+    split_keys = 128          # decode attention: one key split per this many cache positions (at most 32)
+
+    def state_specs(self) -> list[dict]:
+        raise NotImplementedError
+
+    def run(self, tokens: torch.Tensor, sb: SeqBatch) -> torch.Tensor:
+        raise NotImplementedError
+
+    def state_device(self):
+        return next(self.parameters()).device
+
+    def make_cache(self, batch: int, max_len: int, device=None) -> SeqStateCache:
+        cache = SeqStateCache(self.state_specs(), batch, max_len, self.dtype, device or self.state_device())
+        cache.decode_splits = max(1, min(32, max_len // self.split_keys))     # fixed per cache: graph-capturable
+        return cache
+
+    def forward(self, input_ids, position_ids=None, cache=None, kv_lens=None):
+        B, S = input_ids.shape
+        if isinstance(cache, SeqBatch):                   # the engine's packed prefill / decode rows / chunk
+            h = self.run(input_ids.reshape(-1), cache)
+            if cache.decode:
+                cache.desc[2].add_(1)                     # cache.pos[:n], in place (graph-capturable)
+            return h
+        if cache is None:
+            cache = self.make_cache(B, S, input_ids.device)
+        if getattr(cache, "decoding", False) and S == 1:  # generate(): every row one token further
+            sb = cache.head_rows(B)
+            h = self.run(input_ids.reshape(-1), sb)
+            sb.desc[2].add_(1)
+            return h
+        # generate() / plain forward: right-padded prompts, all from the cache's common length
+        lens = [S] * B if kv_lens is None else [int(n) for n in kv_lens.tolist()]
+        start = cache.len
+        sb = SeqBatch.packed(cache, list(range(B)), lens, [start] * B)
+        keep = (torch.arange(S, device=input_ids.device)[None] <
+                torch.tensor(lens, device=input_ids.device)[:, None]).reshape(-1)
+        hp = self.run(input_ids.reshape(-1)[keep], sb)
+        cache.len = start + S
+        if all(n == S for n in lens):
+            return hp
+        h = hp.new_zeros(B * S, hp.shape[1])
+        h[keep] = hp
+        return h
+
+
+class _HeadWeight(nn.Module):
+    def __init__(self, w):
+        super().__init__()
+        self.weight = nn.Parameter(w, requires_grad=False)
+
+
+class SeqStateCausalLM(nn.Module):
+    """``.model`` (a :class:`SeqStateModel`) + ``.lm_head`` like the other causal LMs, so ``infer.generate`` and the
+    serving engine drive it; the engine asks :meth:`make_cache` for its slot pool and :meth:`compute_logits` for
+    logits.  A subclass sets ``config_class`` (``from_pretrained(path)`` / ``from_dict``) and builds ``self.model`` and
+    ``self.lm_head`` from ``(config, weights by checkpoint name, dtype, device)``."""
+
+    config_class = None
+    logit_scale = 1.0
+
+    @classmethod
+    def from_pretrained(cls, path: str, dtype=torch.bfloat16, device=None, **_):
+        import os
+        from safetensors import safe_open
+        cfg = cls.config_class.from_pretrained(path)
+        W = {}
+        for f in sorted(f for f in os.listdir(path) if f.endswith(".safetensors")):
+            with safe_open(os.path.join(path, f), framework="pt", device="cpu") as fh:
+                for k in fh.keys():
+                    W[k] = fh.get_tensor(k)
+        return cls(cfg, W, dtype, device)
+
+    def make_cache(self, batch: int, max_len: int, device=None) -> SeqStateCache:
+        return self.model.make_cache(batch, max_len, device)
+
+    def compute_logits(self, h: torch.Tensor) -> torch.Tensor:
+        """Float logits ``head h * logit_scale`` (bf16 products accumulate in float and are not rounded back)."""
+        w = self.lm_head.weight
+        h2 = h.reshape(-1, h.shape[-1])
+        if w.dtype == torch.float32 or not h2.is_cuda:
+            y = h2.float() @ w.float().t()
+        else:
+            y = torch.mm(h2, w.t(), out_dtype=torch.float32)
+        if self.logit_scale != 1.0:
+            y = y * self.logit_scale
+        return y.view(*h.shape[:-1], w.shape[0])
+
+    def forward(self, input_ids, attention_mask=None, labels=None, past_key_values=None, **_) -> CausalLMOutput:
+        B, S = input_ids.shape
+        kv_lens = attention_mask.sum(1) if attention_mask is not None else None
+        with torch.no_grad():
+            h = self.model(input_ids, None, past_key_values, kv_lens)
+            logits = self.compute_logits(h).view(B, S, -1)
+        loss = None
+        if labels is not None:
+            loss = torch.nn.functional.cross_entropy(logits[:, :-1].reshape(-1, logits.shape[-1]).float(),
+                                                     labels[:, 1:].reshape(-1), ignore_index=-100)
+        return CausalLMOutput(loss=loss, logits=logits, past_key_values=past_key_values)
+
+    @torch.no_grad()
+    def generate(self, input_ids=None, attention_mask=None, generation_config=None, streamer=None, **kw):
+        from ..infer.generate import generate
+        return generate(self, input_ids, attention_mask, generation_config, streamer=streamer, **kw)

@@ -38,7 +38,7 @@ from ..ops.conv import short_conv
 from ..ops.embedding import embed_sincos, sinusoid_inv_freq
 from ..ops.norm import dual_norm_mean, gated_residual_norm, head_norm_gate, rms_norm_f32
 from ..ops.recurrent import decay_gate, gated_delta_scan, mlstm_scan
-from .common import CausalLMOutput, SeqBatch, SeqStateCache
+from .common import SeqBatch, SeqStateCausalLM, SeqStateModel, _HeadWeight
 
 
 @dataclasses.dataclass
@@ -297,7 +297,7 @@ class MobupelLayer(nn.Module):
         return h
 
 
-class MobupelModel(nn.Module):
+class MobupelModel(SeqStateModel):
     def __init__(self, cfg: MobupelConfig, W: dict, dtype, dev):
         super().__init__()
         self.cfg, self.dtype = cfg, dtype
@@ -310,10 +310,8 @@ class MobupelModel(nn.Module):
     def state_specs(self) -> list[dict]:
         return [layer.mix.state_spec() for layer in self.layers]
 
-    def make_cache(self, batch: int, max_len: int, device=None) -> SeqStateCache:
-        cache = SeqStateCache(self.state_specs(), batch, max_len, self.dtype, device or self.embed_tokens.device)
-        cache.decode_splits = max(1, min(32, max_len // 128))     # key splits of decode attention: fixed per cache
-        return cache
+    def state_device(self):
+        return self.embed_tokens.device
 
     def run(self, tokens: torch.Tensor, sb: SeqBatch) -> torch.Tensor:
         """Packed tokens ``[T]`` through all layers; returns the final-normed hidden states ``[T, width]``."""
@@ -327,44 +325,11 @@ class MobupelModel(nn.Module):
                 self.residual_tap.append(x.clone())
         return h
 
-    def forward(self, input_ids, position_ids=None, cache=None, kv_lens=None):
-        B, S = input_ids.shape
-        if isinstance(cache, SeqBatch):                   # the engine's packed prefill / decode rows / chunk
-            h = self.run(input_ids.reshape(-1), cache)
-            if cache.decode:
-                cache.desc[2].add_(1)                     # cache.pos[:n], in place (graph-capturable)
-            return h
-        if cache is None:
-            cache = self.make_cache(B, S, input_ids.device)
-        if getattr(cache, "decoding", False) and S == 1:  # generate(): every row one token further
-            sb = cache.head_rows(B)
-            h = self.run(input_ids.reshape(-1), sb)
-            sb.desc[2].add_(1)
-            return h
-        # generate() / plain forward: right-padded prompts, all from the cache's common length
-        lens = [S] * B if kv_lens is None else [int(n) for n in kv_lens.tolist()]
-        start = cache.len
-        sb = SeqBatch.packed(cache, list(range(B)), lens, [start] * B)
-        keep = (torch.arange(S, device=input_ids.device)[None] <
-                torch.tensor(lens, device=input_ids.device)[:, None]).reshape(-1)
-        hp = self.run(input_ids.reshape(-1)[keep], sb)
-        cache.len = start + S
-        if all(n == S for n in lens):
-            return hp
-        h = hp.new_zeros(B * S, hp.shape[1])
-        h[keep] = hp
-        return h
 
+class MobupelForCausalLM(SeqStateCausalLM):
+    """Mobupel on the shared sequence-state causal-LM frame (``models/common.py``)."""
 
-class _Head(nn.Module):
-    def __init__(self, w):
-        super().__init__()
-        self.weight = nn.Parameter(w, requires_grad=False)
-
-
-class MobupelForCausalLM(nn.Module):
-    """``.model`` + ``.lm_head`` like the other causal LMs, so ``infer.generate`` and the serving engine drive it;
-    the engine asks :meth:`make_cache` for its slot pool and :meth:`compute_logits` for logits."""
+    config_class = MobupelConfig
 
     def __init__(self, cfg: MobupelConfig, weights: dict[str, torch.Tensor], dtype=torch.bfloat16, device=None):
         super().__init__()
@@ -374,50 +339,10 @@ class MobupelForCausalLM(nn.Module):
             raise KeyError(f"Mobupel checkpoint lacks {missing[:6]}")
         self.config = cfg
         self.model = MobupelModel(cfg, weights, dtype, dev)
-        self.lm_head = _Head(weights["head"].to(device=dev, dtype=dtype).contiguous())
+        self.lm_head = _HeadWeight(weights["head"].to(device=dev, dtype=dtype).contiguous())
+        self.logit_scale = cfg.logit_scale
         self.eval()
 
     @classmethod
     def from_config(cls, cfg: MobupelConfig, dtype=torch.bfloat16, device=None, seed: int = 0, rank: int = 16):
         return cls(cfg, random_weights(cfg, seed, rank), dtype, device)
-
-    @classmethod
-    def from_pretrained(cls, path: str, dtype=torch.bfloat16, device=None, **_) -> "MobupelForCausalLM":
-        from safetensors import safe_open
-        cfg = MobupelConfig.from_pretrained(path)
-        W = {}
-        for f in sorted(f for f in os.listdir(path) if f.endswith(".safetensors")):
-            with safe_open(os.path.join(path, f), framework="pt", device="cpu") as fh:
-                for k in fh.keys():
-                    W[k] = fh.get_tensor(k)
-        return cls(cfg, W, dtype, device)
-
-    def make_cache(self, batch: int, max_len: int, device=None) -> SeqStateCache:
-        return self.model.make_cache(batch, max_len, device)
-
-    def compute_logits(self, h: torch.Tensor) -> torch.Tensor:
-        """Float logits ``head h * logit_scale`` (bf16 products accumulate in float and are not rounded back)."""
-        w = self.lm_head.weight
-        h2 = h.reshape(-1, h.shape[-1])
-        if w.dtype == torch.float32 or not h2.is_cuda:
-            y = h2.float() @ w.float().t()
-        else:
-            y = torch.mm(h2, w.t(), out_dtype=torch.float32)
-        return (y * self.config.logit_scale).view(*h.shape[:-1], w.shape[0])
-
-    def forward(self, input_ids, attention_mask=None, labels=None, past_key_values=None, **_) -> CausalLMOutput:
-        B, S = input_ids.shape
-        kv_lens = attention_mask.sum(1) if attention_mask is not None else None
-        with torch.no_grad():
-            h = self.model(input_ids, None, past_key_values, kv_lens)
-            logits = self.compute_logits(h).view(B, S, -1)
-        loss = None
-        if labels is not None:
-            loss = torch.nn.functional.cross_entropy(logits[:, :-1].reshape(-1, logits.shape[-1]).float(),
-                                                     labels[:, 1:].reshape(-1), ignore_index=-100)
-        return CausalLMOutput(loss=loss, logits=logits, past_key_values=past_key_values)
-
-    @torch.no_grad()
-    def generate(self, input_ids=None, attention_mask=None, generation_config=None, streamer=None, **kw):
-        from ..infer.generate import generate
-        return generate(self, input_ids, attention_mask, generation_config, streamer=streamer, **kw)
