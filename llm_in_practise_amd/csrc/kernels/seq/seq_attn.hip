@@ -18,8 +18,8 @@ template <typename T>
 __global__ __launch_bounds__(64) void k_talk_attn_partial(const T* __restrict__ q, int ldq, const T* __restrict__ kc,
                                                           const T* __restrict__ vc, float* __restrict__ pm,
                                                           float* __restrict__ pl, float* __restrict__ pu, int H, int G,
-                                                          int dk, int dv, int max_len, int nsplit, float scale,
-                                                          SeqDesc d) {
+                                                          int dk, int dv, int ldk, int ldv, int max_len, int nsplit,
+                                                          float scale, SeqDesc d) {
   extern __shared__ float sq[];
   const int t = blockIdx.x, g = blockIdx.y, z = blockIdx.z, lane = threadIdx.x;
   const int s = d.tok_seq[t], p = d.tok_pos[t], slot = d.slots[s];
@@ -28,8 +28,8 @@ __global__ __launch_bounds__(64) void k_talk_attn_partial(const T* __restrict__ 
   __syncthreads();
   const int nkeys = p + 1, per = (nkeys + nsplit - 1) / nsplit;
   const int j0 = z * per, j1 = min(nkeys, j0 + per);
-  const T* kbase = kc + ((size_t)slot * max_len) * (G * dk) + kh * dk;
-  const T* vbase = vc + ((size_t)slot * max_len) * GV;
+  const T* kbase = kc + ((size_t)slot * max_len) * ldk + kh * dk;
+  const T* vbase = vc + ((size_t)slot * max_len) * ldv;
   float acc[MAXC];
 #pragma unroll
   for (int c = 0; c < MAXC; ++c) acc[c] = 0.f;
@@ -38,7 +38,7 @@ __global__ __launch_bounds__(64) void k_talk_attn_partial(const T* __restrict__ 
     const int j = jb + lane;
     float sc = -INFINITY;
     if (j < j1) {
-      const T* kr = kbase + (size_t)j * (G * dk);
+      const T* kr = kbase + (size_t)j * ldk;
       float a = 0.f;
       for (int i = 0; i < dk; ++i) a += sq[i] * (float)kr[i];
       sc = a * scale;
@@ -53,7 +53,7 @@ __global__ __launch_bounds__(64) void k_talk_attn_partial(const T* __restrict__ 
     const int cnt = min(64, j1 - jb);
     for (int jj = 0; jj < cnt; ++jj) {
       const float wj = __shfl(w, jj, 64);
-      const T* vr = vbase + (size_t)(jb + jj) * GV;
+      const T* vr = vbase + (size_t)(jb + jj) * ldv;
 #pragma unroll
       for (int c = 0; c < MAXC; ++c) {
         const int col = c * 64 + lane;
@@ -98,8 +98,8 @@ __global__ __launch_bounds__(64 * NW) void k_talk_attn_mfma(const bf16* __restri
                                                        const bf16* __restrict__ vc, float* __restrict__ pm,
                                                        float* __restrict__ pl, float* __restrict__ pu,
                                                        const int* __restrict__ tile_seq, const int* __restrict__ tile_t0,
-                                                       int H, int G, int dk, int dv, int max_len, int nsplit,
-                                                       float scale, SeqDesc d) {
+                                                       int H, int G, int dk, int dv, int ldk, int ldv, int max_len,
+                                                       int nsplit, float scale, SeqDesc d) {
   constexpr int LDMAX = NDT * 32 + 8, LDKMAX = NDS * 16 + 8;
   __shared__ __attribute__((aligned(16))) bf16 sV[32 * LDMAX];
   __shared__ __attribute__((aligned(16))) bf16 sK[NW > 1 ? 32 * LDKMAX : 8];
@@ -114,8 +114,8 @@ __global__ __launch_bounds__(64 * NW) void k_talk_attn_mfma(const bf16* __restri
   const float sl2 = scale * 1.4426950408889634f;   // scores in units of log2: v_exp_f32 is 2^x
   const int trow = 4 * (lane >> 5) + ((lane & 15) >> 2), tcol = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
   const int per = (pmax + nsplit) / nsplit, j0 = z * per, j1 = min(pmax + 1, j0 + per);
-  const bf16* kbase = kc + ((size_t)slot * max_len) * (G * dk) + kh * dk + 8 * hi;
-  const bf16* vbase = vc + ((size_t)slot * max_len) * GV + c * dv;
+  const bf16* kbase = kc + ((size_t)slot * max_len) * ldk + kh * dk + 8 * hi;
+  const bf16* vbase = vc + ((size_t)slot * max_len) * ldv + c * dv;
   bf16x8 qf[NDS];
 #pragma unroll
   for (int ds = 0; ds < NDS; ++ds)
@@ -135,13 +135,13 @@ __global__ __launch_bounds__(64 * NW) void k_talk_attn_mfma(const bf16* __restri
     for (int i = 0; i < VPT; ++i) {
       const int e = threadIdx.x + 64 * NW * i, row = e / vpr, cv = e % vpr;
       if (e < 32 * vpr)
-        pv[i] = *reinterpret_cast<const bf16x8*>(vbase + (size_t)min(jb + row, max_len - 1) * GV + cv * 8);
+        pv[i] = *reinterpret_cast<const bf16x8*>(vbase + (size_t)min(jb + row, max_len - 1) * ldv + cv * 8);
     }
 #pragma unroll
     for (int i = 0; i < KPT; ++i) {
       const int e = threadIdx.x + 64 * NW * i, row = e / kpr, cv = e % kpr;
       if (e < 32 * kpr)
-        pk[i] = *reinterpret_cast<const bf16x8*>(kbase - 8 * hi + (size_t)min(jb + row, max_len - 1) * (G * dk) + cv * 8);
+        pk[i] = *reinterpret_cast<const bf16x8*>(kbase - 8 * hi + (size_t)min(jb + row, max_len - 1) * ldk + cv * 8);
     }
   };
   if (NW > 1 && j0 < j1) fetch(j0);
@@ -164,13 +164,13 @@ __global__ __launch_bounds__(64 * NW) void k_talk_attn_mfma(const bf16* __restri
       for (int e = threadIdx.x; e < 32 * vpr; e += 64) {
         const int row = e / vpr, cv = e % vpr;
         *reinterpret_cast<bf16x8*>(sV + row * LD + cv * 8) =
-            *reinterpret_cast<const bf16x8*>(vbase + (size_t)min(jb + row, max_len - 1) * GV + cv * 8);
+            *reinterpret_cast<const bf16x8*>(vbase + (size_t)min(jb + row, max_len - 1) * ldv + cv * 8);
       }
     }
     f32x16 sc;
 #pragma unroll
     for (int r = 0; r < 16; ++r) sc[r] = 0.f;
-    const bf16* kr = NW > 1 ? sK + ql * LDK + 8 * hi : kbase + (size_t)min(jb + ql, max_len - 1) * (G * dk);
+    const bf16* kr = NW > 1 ? sK + ql * LDK + 8 * hi : kbase + (size_t)min(jb + ql, max_len - 1) * ldk;
 #pragma unroll
     for (int ds = 0; ds < NDS; ++ds)
       if (ds < nds)
@@ -280,33 +280,44 @@ bool seq_attn_mfma_ok(int code, int ldq, int dk, int dv) {
   return code == 0 && dk % 16 == 0 && dk <= 256 && dv % 32 == 0 && dv <= 256 && ldq % 8 == 0;
 }
 
-void seq_talk_attention(int code, const void* q, int ldq, const void* kc, const void* vc, float* pm, float* pl,
-                        float* pu, const float* talk, const void* gate, int ldg, void* out, int H, int G, int dk, int dv,
-                        int max_len, int nsplit, float scale, const int* tile_seq, const int* tile_t0, int ntiles,
-                        SeqDesc d, hipStream_t st) {
+// Pass 1 for any caller: the partial sweeps over a slot-indexed cache whose key rows are ldk and value rows ldv
+// elements apart (values may be columns of the key rows: a latent cache).  Writes pm, pl [T, H, nsplit] and
+// pu [T, H, nsplit, G * dv].
+void seq_attn_sweep(int code, const void* q, int ldq, const void* kc, int ldk, const void* vc, int ldv, float* pm,
+                    float* pl, float* pu, int H, int G, int dk, int dv, int max_len, int nsplit, float scale,
+                    const int* tile_seq, const int* tile_t0, int ntiles, SeqDesc d, hipStream_t st) {
   if (d.Ttot == 0) return;
-  if (tile_seq != nullptr && seq_attn_mfma_ok(code, ldq, dk, dv)) {
+  if (tile_seq != nullptr && seq_attn_mfma_ok(code, ldq, dk, dv) && ldk % 8 == 0 && ldv % 8 == 0) {
     const bool heads = ntiles == d.Ttot && H / G <= 32 && H / G > 1;    // one token per tile: group the heads instead
     const int nw = (!heads && (H / G) % 4 == 0) ? 4 : 1;                 // four heads of a kv head share its tiles
     const dim3 grid(ntiles, heads ? G : H / nw, G * nsplit);
 #define SEQ_ATTN_LAUNCH(NDS, NDT, HEADS, NW)                                                                        \
   hipLaunchKernelGGL((k_talk_attn_mfma<NDS, NDT, HEADS, NW>), grid, dim3(64 * NW), 0, st, (const bf16*)q, ldq,       \
-                     (const bf16*)kc, (const bf16*)vc, pm, pl, pu, tile_seq, tile_t0, H, G, dk, dv, max_len, nsplit, \
-                     scale, d)
+                     (const bf16*)kc, (const bf16*)vc, pm, pl, pu, tile_seq, tile_t0, H, G, dk, dv, ldk, ldv, max_len, \
+                     nsplit, scale, d)
     if (dk <= 128 && dv <= 128) {
       if (heads) SEQ_ATTN_LAUNCH(8, 4, true, 1); else if (nw == 4) SEQ_ATTN_LAUNCH(8, 4, false, 4); else SEQ_ATTN_LAUNCH(8, 4, false, 1);
     } else {
       if (heads) SEQ_ATTN_LAUNCH(16, 8, true, 1); else if (nw == 4) SEQ_ATTN_LAUNCH(16, 8, false, 4); else SEQ_ATTN_LAUNCH(16, 8, false, 1);
     }
 #undef SEQ_ATTN_LAUNCH
-    launch_merge<bf16>(pm, pl, pu, talk, (const bf16*)gate, ldg, (bf16*)out, d.Ttot, H, G, dv, nsplit, st);
     LIPA_CHECK_LAUNCH();
     return;
   }
   SEQ_DISPATCH_T(code, {
     hipLaunchKernelGGL(k_talk_attn_partial<T>, dim3(d.Ttot, H, nsplit), dim3(64), sizeof(float) * dk, st, (const T*)q,
-                       ldq, (const T*)kc, (const T*)vc, pm, pl, pu, H, G, dk, dv, max_len, nsplit, scale, d);
-    launch_merge<T>(pm, pl, pu, talk, (const T*)gate, ldg, (T*)out, d.Ttot, H, G, dv, nsplit, st);
+                       ldq, (const T*)kc, (const T*)vc, pm, pl, pu, H, G, dk, dv, ldk, ldv, max_len, nsplit, scale, d);
   });
+  LIPA_CHECK_LAUNCH();
+}
+
+void seq_talk_attention(int code, const void* q, int ldq, const void* kc, const void* vc, float* pm, float* pl,
+                        float* pu, const float* talk, const void* gate, int ldg, void* out, int H, int G, int dk, int dv,
+                        int max_len, int nsplit, float scale, const int* tile_seq, const int* tile_t0, int ntiles,
+                        SeqDesc d, hipStream_t st) {
+  if (d.Ttot == 0) return;
+  seq_attn_sweep(code, q, ldq, kc, G * dk, vc, G * dv, pm, pl, pu, H, G, dk, dv, max_len, nsplit, scale, tile_seq,
+                 tile_t0, ntiles, d, st);
+  SEQ_DISPATCH_T(code, launch_merge<T>(pm, pl, pu, talk, (const T*)gate, ldg, (T*)out, d.Ttot, H, G, dv, nsplit, st));
   LIPA_CHECK_LAUNCH();
 }

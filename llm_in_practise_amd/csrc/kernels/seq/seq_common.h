@@ -1,6 +1,6 @@
-// Shared pieces of the sequence-state kernels (recurrent mixers, short convolutions, head-mixing attention,
-// fp32-residual norms).  Activations are bf16 or float (template parameter T); the residual stream, every norm,
-// softmax, gate and recurrent state is float.
+// Shared pieces of the sequence-state kernels (recurrent mixers, short convolutions, head-mixing and latent
+// attention, routed experts, fp32-residual norms).  Activations are bf16 or float (template parameter T); the
+// residual stream, every norm, softmax, gate and recurrent state is float.
 //
 // A step's tokens are packed back to back, [Ttot, features].  Sequence b owns tokens seq_off[b] .. seq_off[b+1]-1,
 // lives in state slot slots[b] and starts this step at position pos0[b] (0 = a fresh sequence: its state is taken

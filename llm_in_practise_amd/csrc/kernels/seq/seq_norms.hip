@@ -1,7 +1,8 @@
 // Token-wise kernels of models that keep their residual stream in float: scaled embedding with sinusoidal
 // positions, RMS norms that read float and write the activation type, the gated + normed residual update
-// (fused with the next sublayer's entry norm), the mean of two normed branches, PolyNorm, and the per-head
-// norm + output gate that follows a recurrent mixer.  One 256-thread block per token (one wave per head for the
+// (fused with the next sublayer's entry norm), the mean of two normed branches, PolyNorm, the per-head
+// norm + output gate that follows a recurrent mixer, the token + hashed token-pair embedding, the post-norm residual
+// update, RMS norm of activation rows and the gate-then-grouped-norm of a state-space mixer.  One 256-thread block per token (one wave per head for the
 // head norm); rows are re-read for the second pass (they sit in L1/L2), so any width works.
 #include "seq_common.h"
 
@@ -134,6 +135,149 @@ __global__ __launch_bounds__(256) void k_decay_gate(const float* __restrict__ pr
   g[i] = expf(-expf(a_log[c / dk]) * softplusf_(pre[i] + bias[c]));
 }
 
+// x[t] = table[tok[t]] * scale + pair[(prev * mul_prev + tok[t] * mul_cur) mod buckets]; a sequence's first token takes
+// row `buckets`.  prev is the token before: the packed neighbour, or for a step's first token of a continued
+// sequence the slot's carried token.  The block of a sequence's first token of the step also carries the step's last
+// token into the slot (it alone reads the old one).  Writes the float stream and its copy in the activation type.
+template <typename T>
+__global__ __launch_bounds__(256) void k_embed_pair(const long* __restrict__ tok, const T* __restrict__ table,
+                                                    const T* __restrict__ pair, int* __restrict__ prev_state,
+                                                    float* __restrict__ x, T* __restrict__ h, int W, float scale,
+                                                    long buckets, long mul_prev, long mul_cur, SeqDesc d) {
+  const int t = blockIdx.x, s = d.tok_seq[t], j = t - d.seq_off[s], slot = d.slots[s];
+  const long id = tok[t];
+  long row = buckets;
+  if (pair != nullptr) {
+    if (j > 0)
+      row = (tok[t - 1] * mul_prev + id * mul_cur) % buckets;
+    else if (d.pos0[s] > 0)
+      row = ((long)prev_state[slot] * mul_prev + id * mul_cur) % buckets;
+  }
+  __syncthreads();                                   // every thread has read the carried token
+  if (j == 0 && threadIdx.x == 0 && prev_state != nullptr && !(d.live && !d.live[s]))
+    prev_state[slot] = (int)tok[d.seq_off[s + 1] - 1];
+  for (int c = threadIdx.x; c < W; c += 256) {
+    float v = (float)table[(size_t)id * W + c] * scale;
+    if (pair != nullptr) v += (float)pair[(size_t)row * W + c];
+    x[(size_t)t * W + c] = v;
+    h[(size_t)t * W + c] = (T)v;
+  }
+}
+
+// post-norm residual: x <- rms(alpha x + y) * w in place (float), h = x in the activation type
+template <typename T, typename YT>
+__global__ __launch_bounds__(256) void k_scaled_postnorm(float* __restrict__ x, const YT* __restrict__ y, int ldy,
+                                                         const float* __restrict__ w, T* __restrict__ h, int W,
+                                                         float alpha, float eps) {
+  __shared__ float sc[4];
+  const size_t t = blockIdx.x;
+  float s = 0.f;
+  for (int c = threadIdx.x; c < W; c += 256) {
+    const float v = alpha * x[t * W + c] + (float)y[t * ldy + c];
+    s += v * v;
+  }
+  const float rs = rsqrtf(block_sum256(s, sc) / W + eps);
+  for (int c = threadIdx.x; c < W; c += 256) {
+    const float v = (alpha * x[t * W + c] + (float)y[t * ldy + c]) * rs * w[c];
+    x[t * W + c] = v;
+    h[t * W + c] = (T)v;
+  }
+}
+
+// RMS norm of activation rows (a column slice of a wider matrix is fine)
+template <typename T>
+__global__ __launch_bounds__(256) void k_rms_act(const T* __restrict__ u, int ldu, const float* __restrict__ w,
+                                                 T* __restrict__ out, int n, float eps) {
+  __shared__ float sc[4];
+  const size_t t = blockIdx.x;
+  float s = 0.f;
+  for (int c = threadIdx.x; c < n; c += 256) {
+    const float v = (float)u[t * ldu + c];
+    s += v * v;
+  }
+  const float rs = rsqrtf(block_sum256(s, sc) / n + eps);
+  for (int c = threadIdx.x; c < n; c += 256) out[t * n + c] = (T)((float)u[t * ldu + c] * rs * w[c]);
+}
+
+// gate first, then norm: v = y * silu(z); out = v / rms_part(v) * w, the row cut into equal parts of `gs` entries.
+// VEC: four columns per thread and step (16-byte loads of y and w, 8- or 16-byte loads of z); the gated values of a
+// thread's first two steps stay in registers for the second pass.
+template <typename T>
+__device__ __forceinline__ f32x4 load4_act(const T* p);
+template <>
+__device__ __forceinline__ f32x4 load4_act<float>(const float* p) { return *reinterpret_cast<const f32x4*>(p); }
+template <>
+__device__ __forceinline__ f32x4 load4_act<bf16>(const bf16* p) {
+  const bf16x4 v = *reinterpret_cast<const bf16x4*>(p);
+  return f32x4{(float)v[0], (float)v[1], (float)v[2], (float)v[3]};
+}
+__device__ __forceinline__ void store4_act(float* p, f32x4 v) { *reinterpret_cast<f32x4*>(p) = v; }
+__device__ __forceinline__ void store4_act(bf16* p, f32x4 v) {
+  *reinterpret_cast<bf16x4*>(p) = bf16x4{(bf16)v[0], (bf16)v[1], (bf16)v[2], (bf16)v[3]};
+}
+
+template <typename T, bool VEC>
+__global__ __launch_bounds__(256) void k_gate_group_norm(const float* __restrict__ y, const T* __restrict__ z, int ldz,
+                                                         const float* __restrict__ w, T* __restrict__ out, int n, int gs,
+                                                         float eps) {
+  __shared__ float sc[4];
+  const size_t t = blockIdx.x;
+  const int c0 = blockIdx.y * gs;
+  float s = 0.f;
+  if (VEC) {
+    constexpr int KEEP = 4;                       // steps whose gated values are kept: parts up to 4096 entries
+    f32x4 kept[KEEP];
+#pragma unroll
+    for (int k = 0; k < KEEP; ++k) {
+      const int c = c0 + 4 * threadIdx.x + 1024 * k;
+      kept[k] = f32x4{0.f, 0.f, 0.f, 0.f};
+      if (c < c0 + gs) {
+        const f32x4 g = load4_act<T>(z + t * ldz + c), yv = load4_act<float>(y + t * n + c);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          kept[k][j] = yv[j] * g[j] * sigmoidf_(g[j]);
+          s += kept[k][j] * kept[k][j];
+        }
+      }
+    }
+    for (int c = c0 + 4 * threadIdx.x + 1024 * KEEP; c < c0 + gs; c += 1024) {
+      const f32x4 g = load4_act<T>(z + t * ldz + c), yv = load4_act<float>(y + t * n + c);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float v = yv[j] * g[j] * sigmoidf_(g[j]);
+        s += v * v;
+      }
+    }
+    const float rs = rsqrtf(block_sum256(s, sc) / gs + eps);
+#pragma unroll
+    for (int k = 0; k < KEEP; ++k) {
+      const int c = c0 + 4 * threadIdx.x + 1024 * k;
+      if (c < c0 + gs) {
+        const f32x4 wv = load4_act<float>(w + c);
+        store4_act(out + t * n + c, f32x4{kept[k][0] * rs * wv[0], kept[k][1] * rs * wv[1], kept[k][2] * rs * wv[2],
+                                          kept[k][3] * rs * wv[3]});
+      }
+    }
+    for (int c = c0 + 4 * threadIdx.x + 1024 * KEEP; c < c0 + gs; c += 1024) {
+      const f32x4 g = load4_act<T>(z + t * ldz + c), yv = load4_act<float>(y + t * n + c), wv = load4_act<float>(w + c);
+      f32x4 o;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) o[j] = yv[j] * g[j] * sigmoidf_(g[j]) * rs * wv[j];
+      store4_act(out + t * n + c, o);
+    }
+    return;
+  }
+  for (int c = c0 + threadIdx.x; c < c0 + gs; c += 256) {
+    const float g = (float)z[t * ldz + c], v = y[t * n + c] * g * sigmoidf_(g);
+    s += v * v;
+  }
+  const float rs = rsqrtf(block_sum256(s, sc) / gs + eps);
+  for (int c = c0 + threadIdx.x; c < c0 + gs; c += 256) {
+    const float g = (float)z[t * ldz + c];
+    out[t * n + c] = (T)(y[t * n + c] * g * sigmoidf_(g) * rs * w[c]);
+  }
+}
+
 // ---------------------------------------------------------------------------------------------- launchers
 void seq_embed_sincos(int code, const long* tok, const int* pos, const void* table, const float* inv_freq, float* x,
                       int T_, int W, float scale, hipStream_t st) {
@@ -186,5 +330,50 @@ void seq_decay_gate(const float* pre, const float* bias, const float* a_log, flo
   const size_t n = (size_t)T_ * HD;
   if (n == 0) return;
   hipLaunchKernelGGL(k_decay_gate, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, pre, bias, a_log, g, n, HD, dk);
+  LIPA_CHECK_LAUNCH();
+}
+
+void seq_embed_pair(int code, const long* tok, const void* table, const void* pair, int* prev_state, float* x, void* h,
+                    int W, float scale, long buckets, long mul_prev, long mul_cur, SeqDesc d, hipStream_t st) {
+  if (d.Ttot == 0) return;
+  SEQ_DISPATCH_T(code, hipLaunchKernelGGL(k_embed_pair<T>, dim3(d.Ttot), dim3(256), 0, st, tok, (const T*)table,
+                                          (const T*)pair, prev_state, x, (T*)h, W, scale, buckets, mul_prev, mul_cur, d));
+  LIPA_CHECK_LAUNCH();
+}
+
+void seq_scaled_postnorm(int code, int y_f32, float* x, const void* y, int ldy, const float* w, void* h, int T_, int W,
+                         float alpha, float eps, hipStream_t st) {
+  if (T_ == 0) return;
+  SEQ_DISPATCH_T(code, {
+    if (y_f32)
+      hipLaunchKernelGGL((k_scaled_postnorm<T, float>), dim3(T_), dim3(256), 0, st, x, (const float*)y, ldy, w, (T*)h, W,
+                         alpha, eps);
+    else
+      hipLaunchKernelGGL((k_scaled_postnorm<T, T>), dim3(T_), dim3(256), 0, st, x, (const T*)y, ldy, w, (T*)h, W, alpha,
+                         eps);
+  });
+  LIPA_CHECK_LAUNCH();
+}
+
+void seq_rms_act(int code, const void* u, int ldu, const float* w, void* out, int T_, int n, float eps, hipStream_t st) {
+  if (T_ == 0) return;
+  SEQ_DISPATCH_T(code,
+                 hipLaunchKernelGGL(k_rms_act<T>, dim3(T_), dim3(256), 0, st, (const T*)u, ldu, w, (T*)out, n, eps));
+  LIPA_CHECK_LAUNCH();
+}
+
+void seq_gate_group_norm(int code, const float* y, const void* z, int ldz, const float* w, void* out, int T_, int n,
+                         int parts, float eps, hipStream_t st) {
+  if (T_ == 0) return;
+  const int gs = n / parts;
+  const bool vec = gs % 4 == 0 && n % 4 == 0 && ldz % 4 == 0 && ((uintptr_t)z & 15) == 0;   // 16-byte rows
+  SEQ_DISPATCH_T(code, {
+    if (vec)
+      hipLaunchKernelGGL((k_gate_group_norm<T, true>), dim3(T_, parts), dim3(256), 0, st, y, (const T*)z, ldz, w,
+                         (T*)out, n, gs, eps);
+    else
+      hipLaunchKernelGGL((k_gate_group_norm<T, false>), dim3(T_, parts), dim3(256), 0, st, y, (const T*)z, ldz, w,
+                         (T*)out, n, gs, eps);
+  });
   LIPA_CHECK_LAUNCH();
 }

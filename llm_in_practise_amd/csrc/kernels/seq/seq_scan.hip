@@ -1,5 +1,6 @@
-// Short causal convolutions with carried inputs, and the two matrix-memory recurrences (mLSTM with a running
-// maximum; gated delta rule with a per-channel decay), over packed variable-length sequences with per-slot state.
+// Short causal convolutions with carried inputs, and the matrix-memory recurrences (mLSTM with a running maximum;
+// gated delta rule with a per-channel decay; selective state space with a scalar decay per head), over packed
+// variable-length sequences with per-slot state.
 //
 // Recurrences: every column of the state matrix S[dk, dv] evolves on its own given the step's k, q and gates, so a
 // block owns one (sequence, head) and 256/R columns; a column's dk rows are spread over R adjacent lanes (R a power
@@ -47,8 +48,9 @@ __device__ __forceinline__ float conv_at(const T* __restrict__ u, int ldu, const
 // one wave per (token, head): convolution over time, then the head's activation / norm
 template <typename T, typename OT>
 __global__ __launch_bounds__(64) void k_short_conv(const T* __restrict__ u, int ldu, const float* __restrict__ w,
-                                                   const T* __restrict__ state, OT* __restrict__ out, int C, int taps,
-                                                   ConvArgs a, SeqDesc d, float eps) {
+                                                   const float* __restrict__ bias, const T* __restrict__ state,
+                                                   OT* __restrict__ out, int C, int taps, ConvArgs a, SeqDesc d,
+                                                   float eps) {
   const int t = blockIdx.x, lane = threadIdx.x;
   int hl = blockIdx.y, si = 0;
   while (si < a.nseg - 1 && hl >= a.seg[si].nheads) hl -= a.seg[si++].nheads;
@@ -63,6 +65,7 @@ __global__ __launch_bounds__(64) void k_short_conv(const T* __restrict__ u, int 
     vals[i] = 0.f;
     if (c < sg.hw) {
       float acc = conv_at(u, ldu, state, C, taps, w, t, j, p0, slot, cbase + c);
+      if (bias != nullptr) acc += bias[cbase + c];
       if (sg.mode >= 2) acc = acc * sigmoidf_(acc);
       vals[i] = acc;
       ss += acc * acc;
@@ -363,6 +366,73 @@ __global__ __launch_bounds__(256) void k_delta_scan(const T* __restrict__ q, int
   if (colok) store_rows(Sp, r0, dk, Sr);
 }
 
+// State-space duality form of a selective state space (Mamba-2): per head a scalar decay and step size,
+// dt = softplus(dtraw + dt_bias), S <- exp(-exp(A_log) dt) S + B (dt x)^T, y = S^T C + D x.  S is [N, P] per head, held
+// as [P, N] rows like the other recurrences (key size N = dk, value size P = dv); head hd reads B and C of group
+// hd / (H / G).  The step size and decay of a chunk's tokens are computed in float by the chunk's first lanes.
+template <typename T, int R>
+__global__ __launch_bounds__(256) void k_ssd_scan(const T* __restrict__ q, int ldq, const T* __restrict__ k, int ldk,
+                                                  const T* __restrict__ v, int ldv, const T* __restrict__ dtraw, int lddt,
+                                                  const float* __restrict__ dt_bias, const float* __restrict__ a_log,
+                                                  const float* __restrict__ dskip, float* __restrict__ S,
+                                                  float* __restrict__ out, int H, int G, int dk, int dv, SeqDesc d) {
+  constexpr int DKP = KR * R, NC = 256 / R;
+  __shared__ __attribute__((aligned(16))) float sk[CT * DKP];
+  __shared__ __attribute__((aligned(16))) float sq[CT * DKP];
+  __shared__ float sv[CT * NC];
+  __shared__ float sg[2 * CT];
+  const int s = blockIdx.x / H, hd = blockIdx.x % H, cb = blockIdx.y, tid = threadIdx.x;
+  if (d.live && !d.live[s]) return;
+  const int rg = tid % R, cl = tid / R, col = cb * NC + cl, kh = hd / (H / G), r0 = rg * KR;
+  const bool colok = col < dv;
+  const int t0 = d.seq_off[s], t1 = d.seq_off[s + 1], p0 = d.pos0[s], slot = d.slots[s];
+  float* Sp = S + (((size_t)slot * H + hd) * dv + (colok ? col : 0)) * dk;
+  float Sr[KR];
+  load_rows(Sp, r0, dk, p0 > 0 && colok, Sr);
+  const float rate = expf(a_log[hd]), bias = dt_bias[hd], skip = dskip[hd];
+  float fk[R], fq[R], fv[(16 + R - 1) / R], fdt = 0.f;
+  auto fetch = [&](int c0) {
+    const int n = min(CT, t1 - c0);
+    fetch_rows<T, R>(fk, k + (size_t)c0 * ldk, ldk, kh * dk, dk, n, 1.f, 0.f);
+    fetch_rows<T, R>(fq, q + (size_t)c0 * ldq, ldq, kh * dk, dk, n, 1.f, 0.f);
+    fetch_cols<T, R>(fv, v + (size_t)c0 * ldv, ldv, hd * dv, cb, dv, n);
+    if (tid < n) fdt = (float)dtraw[(size_t)(c0 + tid) * lddt + hd];
+  };
+  if (t0 < t1) fetch(t0);
+  for (int c0 = t0; c0 < t1; c0 += CT) {
+    const int n = min(CT, t1 - c0);
+    __syncthreads();
+    commit_rows<R>(sk, fk);
+    commit_rows<R>(sq, fq);
+    commit_cols<R>(sv, fv);
+    if (tid < n) {
+      const float dt = softplusf_(fdt + bias);
+      sg[2 * tid] = expf(-rate * dt);
+      sg[2 * tid + 1] = dt;
+    }
+    __syncthreads();
+    if (c0 + CT < t1) fetch(c0 + CT);
+    for (int tt = 0; tt < n; ++tt) {
+      const float a = sg[2 * tt], xv = sv[tt * NC + cl], bv = sg[2 * tt + 1] * xv;
+      float num[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int i4 = 0; i4 < KR / 4; ++i4) {
+        const f32x4 kk = *reinterpret_cast<const f32x4*>(sk + tt * DKP + r0 + 4 * i4);
+        const f32x4 qq = *reinterpret_cast<const f32x4*>(sq + tt * DKP + r0 + 4 * i4);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int i = 4 * i4 + j;
+          Sr[i] = a * Sr[i] + kk[j] * bv;
+          num[j] += Sr[i] * qq[j];
+        }
+      }
+      const float y = group_sum<R>((num[0] + num[1]) + (num[2] + num[3]));
+      if (rg == 0 && colok) out[((size_t)(c0 + tt) * H + hd) * dv + col] = y + skip * xv;
+    }
+  }
+  if (colok) store_rows(Sp, r0, dk, Sr);
+}
+
 // ---------------------------------------------------------------------------------------------- launchers
 static int rows_split(int dk) {
   int R = 1;
@@ -384,7 +454,8 @@ int seq_conv_max_taps() { return MAXTAPS; }
   }
 
 // segs: nseg x {c0, nheads, hw, mode}; sw: nseg norm-weight pointers (or null); sscale: nseg scales
-void seq_short_conv(int code, int out_f32, const void* u, int ldu, const float* w, void* state, void* out, int C,
+void seq_short_conv(int code, int out_f32, const void* u, int ldu, const float* w, const float* bias, void* state,
+                    void* out, int C,
                     int taps, int nseg, const int* segs, const float* const* sw, const float* sscale, SeqDesc d,
                     float eps, hipStream_t st) {
   if (d.Ttot == 0) return;
@@ -397,10 +468,10 @@ void seq_short_conv(int code, int out_f32, const void* u, int ldu, const float* 
   }
   SEQ_DISPATCH_T(code, {
     if (out_f32)
-      hipLaunchKernelGGL((k_short_conv<T, float>), dim3(d.Ttot, heads), dim3(64), 0, st, (const T*)u, ldu, w,
+      hipLaunchKernelGGL((k_short_conv<T, float>), dim3(d.Ttot, heads), dim3(64), 0, st, (const T*)u, ldu, w, bias,
                          (const T*)state, (float*)out, C, taps, a, d, eps);
     else
-      hipLaunchKernelGGL((k_short_conv<T, T>), dim3(d.Ttot, heads), dim3(64), 0, st, (const T*)u, ldu, w,
+      hipLaunchKernelGGL((k_short_conv<T, T>), dim3(d.Ttot, heads), dim3(64), 0, st, (const T*)u, ldu, w, bias,
                          (const T*)state, (T*)out, C, taps, a, d, eps);
     if (taps > 1)
       hipLaunchKernelGGL(k_conv_state<T>, dim3(d.B, (C + 255) / 256), dim3(256), 0, st, (const T*)u, ldu, (T*)state, C,
@@ -431,6 +502,20 @@ void seq_delta_scan(int code, const void* q, int ldq, const void* k, int ldk, co
     constexpr int NC = 256 / R;
     hipLaunchKernelGGL((k_delta_scan<T, R>), dim3(d.B * H, (dv + NC - 1) / NC), dim3(256), 0, st, (const T*)q, ldq,
                        (const T*)k, ldk, (const T*)v, ldv, g, bpre, S, out, H, G, dk, dv, d);
+  }));
+  LIPA_CHECK_LAUNCH();
+}
+
+void seq_ssd_scan(int code, const void* q, int ldq, const void* k, int ldk, const void* v, int ldv, const void* dtraw,
+                  int lddt, const float* dt_bias, const float* a_log, const float* dskip, float* S, float* out, int H,
+                  int G, int dk, int dv, SeqDesc d, hipStream_t st) {
+  if (d.B == 0) return;
+  const int Rr = rows_split(dk);
+  SEQ_DISPATCH_T(code, SEQ_DISPATCH_R(Rr, {
+    constexpr int NC = 256 / R;
+    hipLaunchKernelGGL((k_ssd_scan<T, R>), dim3(d.B * H, (dv + NC - 1) / NC), dim3(256), 0, st, (const T*)q, ldq,
+                       (const T*)k, ldk, (const T*)v, ldv, (const T*)dtraw, lddt, dt_bias, a_log, dskip, S, out, H, G,
+                       dk, dv, d);
   }));
   LIPA_CHECK_LAUNCH();
 }

@@ -29,8 +29,32 @@ void seq_polynorm(int, const void*, const float*, void*, int, int, float, hipStr
 void seq_head_norm_gate(int, const float*, const float*, int, const void*, int, const float*, const float*, void*, int,
                         int, int, float, hipStream_t);
 void seq_decay_gate(const float*, const float*, const float*, float*, int, int, int, hipStream_t);
-void seq_short_conv(int, int, const void*, int, const float*, void*, void*, int, int, int, const int*,
+void seq_short_conv(int, int, const void*, int, const float*, const float*, void*, void*, int, int, int, const int*,
                     const float* const*, const float*, SeqDesc, float, hipStream_t);
+void seq_ssd_scan(int, const void*, int, const void*, int, const void*, int, const void*, int, const float*, const float*,
+                  const float*, float*, float*, int, int, int, int, SeqDesc, hipStream_t);
+void seq_embed_pair(int, const long*, const void*, const void*, int*, float*, void*, int, float, long, long, long,
+                    SeqDesc, hipStream_t);
+void seq_scaled_postnorm(int, int, float*, const void*, int, const float*, void*, int, int, float, float, hipStream_t);
+void seq_rms_act(int, const void*, int, const float*, void*, int, int, float, hipStream_t);
+void seq_gate_group_norm(int, const float*, const void*, int, const float*, void*, int, int, int, float, hipStream_t);
+void seq_attn_sweep(int, const void*, int, const void*, int, const void*, int, float*, float*, float*, int, int, int,
+                    int, int, int, float, const int*, const int*, int, SeqDesc, hipStream_t);
+void seq_latent_kv_store(int, const void*, int, const float*, const float*, void*, int, int, int, int, float, SeqDesc,
+                         hipStream_t);
+void seq_latent_q_assemble(int, const void*, size_t, size_t, const void*, int, int, const float*, void*, int, int, int,
+                           int, SeqDesc, hipStream_t);
+void seq_latent_merge(int, const float*, const float*, const float*, const void*, int, void*, int, int, int, int,
+                      hipStream_t);
+void seq_route_grouped(const float*, const float*, int*, float*, int, int, int, int, int, float, hipStream_t);
+void seq_route_fused(int, const void*, int, const float*, const float*, int*, float*, int, int, int, int, int, int, float,
+                     hipStream_t);
+void seq_moe_pairs(int, const void*, int, const void*, const void*, const int*, const float*, const void*, void*, float*,
+                   int, int, int, int, int, float, hipStream_t);
+void seq_moe_combine(int, const void*, const long*, const int*, const float*, const void*, int, const void*, float*, int,
+                     int, int, int, hipStream_t);
+void seq_ff_act(int, const void*, void*, int, int, int, float, hipStream_t);
+int seq_route_max_outputs();
 void seq_mlstm_scan(int, const void*, int, const void*, int, const void*, int, const float*, const float*, const float*,
                     const float*, float, float, float*, float*, float*, float*, float*, float*, int, int, int, SeqDesc,
                     hipStream_t);
@@ -191,7 +215,7 @@ Tensor decay_gate(Tensor pre, Tensor bias, Tensor a_log, int64_t dk) {
 // (updated in place), segs = [[c0, heads, head width, mode]...], seg_w / seg_scale per segment.
 Tensor short_conv(Tensor u, Tensor w, optional<Tensor> state, std::vector<std::vector<int64_t>> segs,
                   std::vector<optional<Tensor>> seg_w, std::vector<double> seg_scale, std::vector<Tensor> desc,
-                  optional<Tensor> live, double eps, bool out_f32) {
+                  optional<Tensor> live, double eps, bool out_f32, optional<Tensor> bias) {
   const int code = code_of(u);
   TORCH_CHECK(u.dim() == 2, "u: [T, C]");
   const int64_t T = u.size(0), C = u.size(1);
@@ -200,6 +224,12 @@ Tensor short_conv(Tensor u, Tensor w, optional<Tensor> state, std::vector<std::v
   TORCH_CHECK(w.dim() == 2 && w.size(0) == C, "conv weight: [C, taps]");
   const int taps = (int)w.size(1);
   TORCH_CHECK(taps >= 1 && taps <= seq_conv_max_taps(), "conv taps out of range");
+  const float* bp = nullptr;
+  if (bias && bias->defined()) {
+    f32c(*bias, "conv bias");
+    TORCH_CHECK(bias->numel() == C, "conv bias: [C]");
+    bp = bias->data_ptr<float>();
+  }
   SeqDesc d = desc_of(desc, live, T);
   void* sp = nullptr;
   if (taps > 1) {
@@ -230,7 +260,7 @@ Tensor short_conv(Tensor u, Tensor w, optional<Tensor> state, std::vector<std::v
   }
   TORCH_CHECK(c == C, "segments must cover all channels");
   auto out = at::empty({T, C}, u.options().dtype(out_f32 ? at::kFloat : u.scalar_type()));
-  seq_short_conv(code, out_f32 ? 1 : 0, u.data_ptr(), ld(u), w.data_ptr<float>(), sp, out.data_ptr(), (int)C, taps, nseg,
+  seq_short_conv(code, out_f32 ? 1 : 0, u.data_ptr(), ld(u), w.data_ptr<float>(), bp, sp, out.data_ptr(), (int)C, taps, nseg,
                  flat, wp, sc, d, (float)eps, stream());
   return out;
 }
@@ -339,6 +369,284 @@ Tensor talk_attention(Tensor q, Tensor kc, Tensor vc, Tensor talk, Tensor gate, 
   return out;
 }
 
+// ---- selective state space (state-space duality form): q = C, k = B [T, G * N], v = x [T, H * P], dtraw [T, H]
+Tensor ssd_scan(Tensor q, Tensor k, Tensor v, Tensor dtraw, Tensor dt_bias, Tensor a_log, Tensor dskip, Tensor S,
+                int64_t H, int64_t G, std::vector<Tensor> desc, optional<Tensor> live) {
+  const int code = code_of(q);
+  const int64_t T = q.size(0);
+  TORCH_CHECK(G >= 1 && H % G == 0 && q.dim() == 2 && q.size(1) % G == 0 && v.dim() == 2 && v.size(1) % H == 0,
+              "q/k: [T, G * N], v: [T, H * P]");
+  const int64_t dk = q.size(1) / G, dv = v.size(1) / H;
+  rows(q, T, G * dk, code, "C");
+  rows(k, T, G * dk, code, "B");
+  rows(v, T, H * dv, code, "x");
+  rows(dtraw, T, H, code, "dt");
+  f32c(dt_bias, "dt_bias");
+  f32c(a_log, "A_log");
+  f32c(dskip, "D");
+  TORCH_CHECK(dt_bias.numel() == H && a_log.numel() == H && dskip.numel() == H, "per-head constants: [H]");
+  TORCH_CHECK(dk <= seq_scan_max_dk(), "state size above ", seq_scan_max_dk());
+  check_state(S, H, dv, dk);
+  SeqDesc d = desc_of(desc, live, T);
+  auto out = at::empty({T, H * dv}, S.options());
+  seq_ssd_scan(code, q.data_ptr(), ld(q), k.data_ptr(), ld(k), v.data_ptr(), ld(v), dtraw.data_ptr(), ld(dtraw),
+               dt_bias.data_ptr<float>(), a_log.data_ptr<float>(), dskip.data_ptr<float>(), S.data_ptr<float>(),
+               out.data_ptr<float>(), (int)H, (int)G, (int)dk, (int)dv, d, stream());
+  return out;
+}
+
+// returns {x float [T, W], h activation copy}; prev [slots] int32 (the token before a continued step), pair table
+// [buckets + 1, W] or none
+std::vector<Tensor> embed_pair(Tensor tok, Tensor table, optional<Tensor> pair, optional<Tensor> prev, double scale,
+                               int64_t mul_prev, int64_t mul_cur, std::vector<Tensor> desc, optional<Tensor> live) {
+  TORCH_CHECK(tok.is_cuda() && tok.scalar_type() == at::kLong && tok.is_contiguous(), "tokens: int64");
+  TORCH_CHECK(table.is_cuda() && table.is_contiguous() && table.dim() == 2, "table");
+  const int code = code_of(table);
+  const int64_t T = tok.numel(), W = table.size(1);
+  SeqDesc d = desc_of(desc, live, T);
+  const void* pp = nullptr;
+  int* sp = nullptr;
+  long buckets = 0;
+  if (pair && pair->defined()) {
+    TORCH_CHECK(pair->is_cuda() && pair->is_contiguous() && pair->dim() == 2 && pair->size(1) == W &&
+                    pair->size(0) >= 2 && code_of(*pair) == code, "pair table: [buckets + 1, W]");
+    TORCH_CHECK(prev && prev->defined() && prev->is_cuda() && prev->scalar_type() == at::kInt && prev->is_contiguous(),
+                "carried tokens: int32 [slots]");
+    TORCH_CHECK(mul_prev >= 0 && mul_cur >= 0, "multipliers must not be negative");
+    pp = pair->data_ptr();
+    sp = prev->data_ptr<int>();
+    buckets = pair->size(0) - 1;
+  }
+  auto x = at::empty({T, W}, table.options().dtype(at::kFloat));
+  auto h = at::empty({T, W}, table.options());
+  seq_embed_pair(code, tok.data_ptr<long>(), table.data_ptr(), pp, sp, x.data_ptr<float>(), h.data_ptr(), (int)W,
+                 (float)scale, buckets, (long)mul_prev, (long)mul_cur, d, stream());
+  return {x, h};
+}
+
+// x (float, in place) <- rms(alpha x + y) * w; returns its copy in the activation type (bf16 when out_bf16)
+Tensor scaled_postnorm(Tensor x, Tensor y, Tensor w, double alpha, double eps, bool out_bf16) {
+  f32c(x, "x");
+  f32c(w, "w");
+  const int W = (int)x.size(-1), T = (int)(x.numel() / W), code = out_bf16 ? 0 : 1;
+  const bool yf = y.scalar_type() == at::kFloat;
+  TORCH_CHECK(w.numel() == W, "norm weight size");
+  TORCH_CHECK(y.is_cuda() && y.dim() == 2 && y.size(0) == T && y.size(1) == W && (T == 0 || y.stride(1) == 1) &&
+                  (yf || code_of(y) == code), "y: [T, W], float or the activation type");
+  auto h = at::empty({T, W}, x.options().dtype(out_bf16 ? at::kBFloat16 : at::kFloat));
+  seq_scaled_postnorm(code, yf ? 1 : 0, x.data_ptr<float>(), y.data_ptr(), ld(y), w.data_ptr<float>(), h.data_ptr(), T,
+                      W, (float)alpha, (float)eps, stream());
+  return h;
+}
+
+Tensor rms_act(Tensor u, Tensor w, double eps) {
+  const int code = code_of(u);
+  TORCH_CHECK(u.dim() == 2, "u: [T, n]");
+  const int64_t T = u.size(0), n = u.size(1);
+  rows(u, T, n, code, "u");
+  f32c(w, "w");
+  TORCH_CHECK(w.numel() == n, "norm weight size");
+  auto out = at::empty({T, n}, u.options());
+  seq_rms_act(code, u.data_ptr(), ld(u), w.data_ptr<float>(), out.data_ptr(), (int)T, (int)n, (float)eps, stream());
+  return out;
+}
+
+Tensor gate_group_norm(Tensor y, Tensor z, Tensor w, int64_t parts, double eps) {
+  f32c(y, "y");
+  TORCH_CHECK(y.dim() == 2, "y: [T, n]");
+  const int64_t T = y.size(0), n = y.size(1);
+  const int code = code_of(z);
+  rows(z, T, n, code, "z");
+  f32c(w, "w");
+  TORCH_CHECK(w.numel() == n && parts >= 1 && parts <= 65535 && n % parts == 0, "norm weight [n]; parts must divide n");
+  auto out = at::empty({T, n}, z.options());
+  seq_gate_group_norm(code, y.data_ptr<float>(), z.data_ptr(), ld(z), w.data_ptr<float>(), out.data_ptr(), (int)T, (int)n,
+                      (int)parts, (float)eps, stream());
+  return out;
+}
+
+// ---- latent attention over a cache of rows [c (R) | rotated shared key part (dr)]
+static void check_latent_cache(const Tensor& cache, int64_t R, int64_t dr, int code) {
+  TORCH_CHECK(cache.is_cuda() && cache.is_contiguous() && cache.dim() == 3 && cache.size(2) == R + dr &&
+                  code_of(cache) == code, "latent cache: [slots, max_len, kv_rank + rot_dim]");
+}
+static void check_freq(const Tensor& f, int64_t dims, int64_t dr) {
+  f32c(f, "inv_freq");
+  TORCH_CHECK(dims >= 0 && dims % 2 == 0 && dims <= dr && f.numel() * 2 >= dims, "rotation: even dims <= rot_dim");
+}
+
+void latent_kv_store(Tensor u, Tensor w, Tensor inv_freq, Tensor cache, int64_t dims, double eps,
+                     std::vector<Tensor> desc) {
+  const int code = code_of(u);
+  TORCH_CHECK(u.dim() == 2, "u: [T, kv_rank + rot_dim]");
+  const int64_t T = u.size(0), R = w.numel(), dr = u.size(1) - R;
+  TORCH_CHECK(dr >= 0, "down-projection narrower than the latent");
+  rows(u, T, R + dr, code, "u");
+  f32c(w, "w");
+  check_freq(inv_freq, dims, dr);
+  check_latent_cache(cache, R, dr, code);
+  SeqDesc d = desc_of(desc, optional<Tensor>(), T);
+  seq_latent_kv_store(code, u.data_ptr(), ld(u), w.data_ptr<float>(), inv_freq.data_ptr<float>(), cache.data_ptr(),
+                      (int)R, (int)dr, (int)dims, (int)cache.size(1), (float)eps, d, stream());
+}
+
+// qa [H, T, R] (any strides with unit inner stride): the unrotated query parts already multiplied by W_uk;
+// q [T, H * (dn + dr)]; gate [T, H] pre-activations or none.  Returns [T, H, R]: gate * softmax-weighted latents.
+Tensor latent_attention(Tensor qa, Tensor q, Tensor cache, optional<Tensor> gate, Tensor inv_freq, int64_t H, int64_t dn,
+                        int64_t dims, double scale, int64_t nsplit, std::vector<Tensor> desc, std::vector<Tensor> tiles) {
+  const int code = code_of(q);
+  const int64_t T = q.size(0);
+  TORCH_CHECK(qa.is_cuda() && qa.dim() == 3 && qa.size(0) == H && qa.size(1) == T && (qa.numel() == 0 || qa.stride(2) == 1) &&
+                  code_of(qa) == code, "qa: [H, T, kv_rank]");
+  const int64_t R = qa.size(2);
+  TORCH_CHECK(q.dim() == 2 && q.size(1) % H == 0 && q.size(1) / H >= dn, "q: [T, H * (dim + rot_dim)]");
+  const int64_t dr = q.size(1) / H - dn;
+  rows(q, T, H * (dn + dr), code, "q");
+  check_freq(inv_freq, dims, dr);
+  check_latent_cache(cache, R, dr, code);
+  TORCH_CHECK(R <= seq_attn_max_cols(), "attention: kv_rank above ", seq_attn_max_cols());
+  TORCH_CHECK(nsplit >= 1 && nsplit <= 1024, "nsplit");
+  const void* gp = nullptr;
+  int ldg = 0;
+  if (gate && gate->defined()) {
+    rows(*gate, T, H, code, "gate");
+    gp = gate->data_ptr();
+    ldg = ld(*gate);
+  }
+  SeqDesc d = desc_of(desc, optional<Tensor>(), T);
+  const int* tseq = nullptr;
+  const int* tt0 = nullptr;
+  int ntiles = 0;
+  if (tiles.size() == 2) {
+    for (auto& t : tiles) TORCH_CHECK(t.is_cuda() && t.scalar_type() == at::kInt && t.is_contiguous(), "tiles: int32");
+    TORCH_CHECK(tiles[0].numel() == tiles[1].numel(), "tiles: two arrays of one length");
+    tseq = tiles[0].data_ptr<int>();
+    tt0 = tiles[1].data_ptr<int>();
+    ntiles = (int)tiles[0].numel();
+    TORCH_CHECK((int64_t)ntiles * 32 >= T && nsplit <= 65535, "tiles must cover the tokens");
+  }
+  auto fo = q.options().dtype(at::kFloat);
+  auto Q = at::empty({T, H * (R + dr)}, q.options());
+  auto pm = at::empty({T, H, nsplit}, fo), pl = at::empty({T, H, nsplit}, fo), pu = at::empty({T, H, nsplit, R}, fo);
+  auto out = at::empty({T, H, R}, q.options());
+  seq_latent_q_assemble(code, qa.data_ptr(), (size_t)qa.stride(0), (size_t)qa.stride(1), q.data_ptr(), ld(q), (int)dn,
+                        inv_freq.data_ptr<float>(), Q.data_ptr(), (int)H, (int)R, (int)dr, (int)dims, d, stream());
+  seq_attn_sweep(code, Q.data_ptr(), (int)(H * (R + dr)), cache.data_ptr(), (int)(R + dr), cache.data_ptr(),
+                 (int)(R + dr), pm.data_ptr<float>(), pl.data_ptr<float>(), pu.data_ptr<float>(), (int)H, 1,
+                 (int)(R + dr), (int)R, (int)cache.size(1), (int)nsplit, (float)scale, tseq, tt0, ntiles, d, stream());
+  seq_latent_merge(code, pm.data_ptr<float>(), pl.data_ptr<float>(), pu.data_ptr<float>(), gp, ldg, out.data_ptr(),
+                   (int)T, (int)H, (int)R, (int)nsplit, stream());
+  return out;
+}
+
+// ---- mixture of experts
+static const float* check_routing(int64_t n, const optional<Tensor>& corr, int64_t top, int64_t groups, int64_t keep) {
+  TORCH_CHECK(n >= 1 && n <= seq_route_max_outputs(), "router outputs above ", seq_route_max_outputs());
+  TORCH_CHECK(top >= 1 && top <= n, "top");
+  TORCH_CHECK(groups >= 1 && groups <= 64 && n % groups == 0 && keep >= 1 && keep <= groups, "groups must divide n");
+  TORCH_CHECK(top <= keep * (n / groups), "fewer eligible outputs than `top`");
+  if (corr && corr->defined()) {
+    f32c(*corr, "correction");
+    TORCH_CHECK(corr->numel() == n, "correction: [n]");
+    return corr->data_ptr<float>();
+  }
+  return nullptr;
+}
+
+std::vector<Tensor> route_grouped(Tensor z, optional<Tensor> corr, int64_t top, int64_t groups, int64_t keep,
+                                  double scale) {
+  f32c(z, "router logits");
+  TORCH_CHECK(z.dim() == 2, "router logits: [T, n]");
+  const int64_t T = z.size(0), n = z.size(1);
+  const float* cp = check_routing(n, corr, top, groups, keep);
+  auto idx = at::empty({T, top}, z.options().dtype(at::kInt));
+  auto w = at::empty({T, top}, z.options());
+  seq_route_grouped(z.data_ptr<float>(), cp, idx.data_ptr<int>(), w.data_ptr<float>(), (int)T, (int)n, (int)top,
+                    (int)groups, (int)keep, (float)scale, stream());
+  return {idx, w};
+}
+
+// the router product (float weights [n, W], activations h [T, W] as they are, float accumulation) and the routing
+std::vector<Tensor> route_fused(Tensor h, Tensor router, optional<Tensor> corr, int64_t top, int64_t groups,
+                                int64_t keep, double scale) {
+  const int code = code_of(h);
+  TORCH_CHECK(h.dim() == 2, "h: [T, W]");
+  const int64_t T = h.size(0), W = h.size(1);
+  rows(h, T, W, code, "h");
+  f32c(router, "router");
+  TORCH_CHECK(router.dim() == 2 && router.size(1) == W, "router: [n, W]");
+  const int64_t n = router.size(0);
+  const float* cp = check_routing(n, corr, top, groups, keep);
+  auto idx = at::empty({T, top}, h.options().dtype(at::kInt));
+  auto w = at::empty({T, top}, h.options().dtype(at::kFloat));
+  seq_route_fused(code, h.data_ptr(), ld(h), router.data_ptr<float>(), cp, idx.data_ptr<int>(), w.data_ptr<float>(),
+                  (int)T, (int)n, (int)W, (int)top, (int)groups, (int)keep, (float)scale, stream());
+  return {idx, w};
+}
+
+static void check_route(const Tensor& idx, const Tensor& w, int64_t T) {
+  TORCH_CHECK(idx.is_cuda() && idx.scalar_type() == at::kInt && idx.is_contiguous() && idx.dim() == 2 && idx.size(0) == T,
+              "expert ids: int32 [T, top]");
+  f32c(w, "weights");
+  TORCH_CHECK(w.sizes() == idx.sizes(), "weights: [T, top]");
+}
+
+// few tokens: every (token, expert) pair streams its expert.  wgu [E, 2, F, W], wd [E, W, F]; returns float [T, W]
+Tensor moe_pairs(Tensor h, Tensor wgu, Tensor wd, Tensor idx, Tensor w, optional<Tensor> shared, double limit) {
+  const int code = code_of(h);
+  TORCH_CHECK(h.is_cuda() && h.dim() == 2 && h.is_contiguous(), "h: [T, W] contiguous");
+  const int64_t T = h.size(0), W = h.size(1);
+  TORCH_CHECK(wgu.is_cuda() && wgu.is_contiguous() && wgu.dim() == 4 && wgu.size(1) == 2 && wgu.size(3) == W &&
+                  code_of(wgu) == code, "wgu: [E, 2, F, W]");
+  const int64_t E = wgu.size(0), F = wgu.size(2);
+  TORCH_CHECK(wd.is_cuda() && wd.is_contiguous() && wd.dim() == 3 && wd.size(0) == E && wd.size(1) == W &&
+                  wd.size(2) == F && code_of(wd) == code, "wd: [E, W, F]");
+  check_route(idx, w, T);
+  const int64_t top = idx.size(1);
+  const void* sp = nullptr;
+  if (shared && shared->defined()) {
+    TORCH_CHECK(shared->is_cuda() && shared->is_contiguous() && shared->dim() == 2 && shared->size(0) == T &&
+                    shared->size(1) == W && code_of(*shared) == code, "shared: [T, W]");
+    sp = shared->data_ptr();
+  }
+  TORCH_CHECK(T * top <= 65535 && T <= 65535, "the pairs path is for few tokens");
+  auto a = at::empty({T * top, F}, h.options());
+  auto out = at::empty({T, W}, h.options().dtype(at::kFloat));
+  seq_moe_pairs(code, h.data_ptr(), (int)W, wgu.data_ptr(), wd.data_ptr(), idx.data_ptr<int>(), w.data_ptr<float>(), sp,
+                a.data_ptr(), out.data_ptr<float>(), (int)T, (int)top, (int)E, (int)F, (int)W, (float)limit, stream());
+  return out;
+}
+
+// ys [rows, W]: expert outputs in expert-sorted order; pos [T, top] int64: the row of every pair
+Tensor moe_combine_sorted(Tensor ys, Tensor pos, Tensor idx, Tensor w, Tensor h, optional<Tensor> shared, int64_t E) {
+  const int code = code_of(h);
+  TORCH_CHECK(h.is_cuda() && h.dim() == 2 && h.is_contiguous(), "h: [T, W] contiguous");
+  const int64_t T = h.size(0), W = h.size(1);
+  check_route(idx, w, T);
+  TORCH_CHECK(ys.is_cuda() && ys.is_contiguous() && ys.dim() == 2 && ys.size(1) == W && code_of(ys) == code, "ys: [rows, W]");
+  TORCH_CHECK(pos.is_cuda() && pos.scalar_type() == at::kLong && pos.is_contiguous() && pos.numel() == idx.numel(),
+              "pos: int64 [T, top]");
+  const void* sp = nullptr;
+  if (shared && shared->defined()) {
+    TORCH_CHECK(shared->is_cuda() && shared->is_contiguous() && shared->dim() == 2 && shared->size(0) == T &&
+                    shared->size(1) == W && code_of(*shared) == code, "shared: [T, W]");
+    sp = shared->data_ptr();
+  }
+  auto out = at::empty({T, W}, h.options().dtype(at::kFloat));
+  seq_moe_combine(code, ys.data_ptr(), pos.data_ptr<long>(), idx.data_ptr<int>(), w.data_ptr<float>(), h.data_ptr(),
+                  (int)W, sp, out.data_ptr<float>(), (int)T, (int)idx.size(1), (int)E, (int)W, stream());
+  return out;
+}
+
+// mode 0: tanh-form GELU of z [T, F]; mode 1: clipped GLU of z [T, 2F] = [gate | up]
+Tensor ff_act(Tensor z, int64_t mode, double limit) {
+  TORCH_CHECK(z.is_cuda() && z.is_contiguous() && z.dim() == 2 && (mode == 0 || (mode == 1 && z.size(1) % 2 == 0)), "z");
+  const int64_t T = z.size(0), F = mode == 0 ? z.size(1) : z.size(1) / 2;
+  auto out = at::empty({T, F}, z.options());
+  seq_ff_act(code_of(z), z.data_ptr(), out.data_ptr(), (int)T, (int)F, (int)mode, (float)limit, stream());
+  return out;
+}
+
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("embed_sincos", &embed_sincos);
   m.def("rms_f32", &rms_f32);
@@ -347,8 +655,22 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("polynorm", &polynorm);
   m.def("head_norm_gate", &head_norm_gate);
   m.def("decay_gate", &decay_gate);
-  m.def("short_conv", &short_conv);
+  m.def("short_conv", &short_conv, py::arg("u"), py::arg("w"), py::arg("state"), py::arg("segs"), py::arg("seg_w"),
+        py::arg("seg_scale"), py::arg("desc"), py::arg("live"), py::arg("eps"), py::arg("out_f32"),
+        py::arg("bias") = py::none());
   m.def("mlstm_scan", &mlstm_scan);
   m.def("delta_scan", &delta_scan);
   m.def("talk_attention", &talk_attention);
+  m.def("ssd_scan", &ssd_scan);
+  m.def("embed_pair", &embed_pair);
+  m.def("scaled_postnorm", &scaled_postnorm);
+  m.def("rms_act", &rms_act);
+  m.def("gate_group_norm", &gate_group_norm);
+  m.def("latent_kv_store", &latent_kv_store);
+  m.def("latent_attention", &latent_attention);
+  m.def("route_grouped", &route_grouped);
+  m.def("route_fused", &route_fused);
+  m.def("moe_pairs", &moe_pairs);
+  m.def("moe_combine_sorted", &moe_combine_sorted);
+  m.def("ff_act", &ff_act);
 }

@@ -56,3 +56,21 @@ def polynorm(z: torch.Tensor, coef: torch.Tensor, eps: float) -> torch.Tensor:
     if use_seq(z):
         return native_seq().polynorm(z.contiguous(), coef, eps)
     return ref.polynorm(z, coef, eps)
+
+
+def gelu_tanh(z: torch.Tensor) -> torch.Tensor:
+    """The tanh form of GELU on a matrix-product output (serving path, no autograd)."""
+    from . import reference as ref
+    from ._native import native_seq, use_seq
+    if use_seq(z):
+        return native_seq().ff_act(z.contiguous(), 0, 0.0)
+    return ref.gelu_tanh(z)
+
+
+def clipped_glu(z: torch.Tensor, limit: float) -> torch.Tensor:
+    """``z = [gate | up]``: ``g = min(gate, limit)``, ``u = clamp(up, -limit, limit)``, ``g * sigmoid(1.702 g) * (u + 1)``."""
+    from . import reference as ref
+    from ._native import native_seq, use_seq
+    if use_seq(z):
+        return native_seq().ff_act(z.contiguous(), 1, limit)
+    return ref.clipped_glu(z, limit)

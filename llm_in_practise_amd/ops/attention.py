@@ -169,3 +169,35 @@ def talking_heads_attention(q, k_cache, v_cache, talk, gate_pre, heads: int, kv_
         return native_seq().talk_attention(q, k_cache, v_cache, talk, gate_pre, heads, kv_heads, scale, nsplit, sb.desc,
                                            sb.tiles)
     return ref.talk_attention(q, k_cache, v_cache, talk, gate_pre, heads, kv_heads, scale, sb)
+
+
+def rotary_inv_freq(dims: int, base: float) -> torch.Tensor:
+    """``base^(-2i / dims)`` for i < dims / 2, evaluated in float64 and rounded once to float."""
+    i = torch.arange(dims // 2, dtype=torch.float64)
+    return (float(base) ** (-2.0 * i / max(dims, 1))).float()
+
+
+def latent_kv_store(u: torch.Tensor, norm_weight: torch.Tensor, inv_freq: torch.Tensor, cache: torch.Tensor,
+                    rot_dims: int, eps: float, sb) -> None:
+    """Writes a step's rows of a latent attention cache ``[slots, max_len, R + dr]``: ``u`` ``[T, R + dr]`` is the
+    down-projection; its first ``R`` entries are RMS-normed (``norm_weight``), its last ``dr`` are the key part shared
+    by all heads, rotated pairwise (neighbours ``2i, 2i+1`` below ``rot_dims``) at each token's position."""
+    from ._native import native_seq, use_seq
+    if use_seq(u):
+        return native_seq().latent_kv_store(u, norm_weight, inv_freq, cache, rot_dims, eps, sb.desc)
+    return ref.latent_kv_store(u, norm_weight, inv_freq, cache, rot_dims, eps, sb)
+
+
+def latent_attention(q_abs: torch.Tensor, q: torch.Tensor, cache: torch.Tensor, gate_pre: torch.Tensor | None,
+                     inv_freq: torch.Tensor, heads: int, dim: int, rot_dims: int, scale: float, sb,
+                     nsplit: int = 1) -> torch.Tensor:
+    """Causal softmax attention of ``heads`` query heads over ONE shared row per key position, ``[c | kr]``:
+    ``score_h = (q_abs_h . c + rot(q_rot_h) . kr) * scale``, result ``sum_j w_h(j) c(j)`` times
+    ``sigmoid(gate_pre[t, h])``.  ``q_abs`` ``[H, T, R]`` holds the unrotated query parts already carried through the
+    key up-projection; ``q`` ``[T, H*(dim + dr)]`` supplies the rotated parts (rotated here).  Returns ``[T, H, R]``;
+    the caller applies the value up-projection.  Scores and weights are float."""
+    from ._native import native_seq, use_seq
+    if use_seq(q):
+        return native_seq().latent_attention(q_abs, q, cache, gate_pre, inv_freq, heads, dim, rot_dims, scale, nsplit,
+                                             sb.desc, sb.tiles)
+    return ref.latent_attention(q_abs, q, cache, gate_pre, inv_freq, heads, dim, rot_dims, scale, sb)

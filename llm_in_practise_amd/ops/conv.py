@@ -19,12 +19,13 @@ PLAIN, RMS, SILU, SILU_UNIT = 0, 1, 2, 3
 
 
 def short_conv(u: torch.Tensor, weight: torch.Tensor, state: torch.Tensor | None, segments, sb, eps: float,
-               out_f32: bool = False) -> torch.Tensor:
+               out_f32: bool = False, bias: torch.Tensor | None = None) -> torch.Tensor:
     """``u`` ``[T, C]`` (a column slice of a wider matrix is fine), ``weight`` float ``[C, taps]``, ``segments`` a list
-    of ``(first channel, heads, head width, mode, norm weight | None, scale)``, ``sb`` the step's ``SeqBatch``."""
+    of ``(first channel, heads, head width, mode, norm weight | None, scale)``, ``sb`` the step's ``SeqBatch``;
+    ``bias`` float ``[C]`` is added before the segment's activation."""
     segs = [[int(s[0]), int(s[1]), int(s[2]), int(s[3])] for s in segments]
     sw = [s[4] for s in segments]
     sc = [float(s[5]) for s in segments]
     if use_seq(u):
-        return native_seq().short_conv(u, weight, state, segs, sw, sc, sb.desc, sb.live, eps, out_f32)
-    return ref.short_conv(u, weight, state, segs, sw, sc, sb, eps, out_f32)
+        return native_seq().short_conv(u, weight, state, segs, sw, sc, sb.desc, sb.live, eps, out_f32, bias)
+    return ref.short_conv(u, weight, state, segs, sw, sc, sb, eps, out_f32, bias)

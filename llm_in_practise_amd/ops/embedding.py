@@ -120,3 +120,17 @@ def embed_sincos(tokens: torch.Tensor, positions: torch.Tensor, table: torch.Ten
         return native_seq().embed_sincos(tokens.reshape(-1).long().contiguous(),
                                          positions.reshape(-1).int().contiguous(), table, inv_freq, scale)
     return ref.embed_sincos(tokens, positions, table, inv_freq, scale)
+
+
+def embed_pair(tokens: torch.Tensor, table: torch.Tensor, pair_table: torch.Tensor | None, prev: torch.Tensor | None,
+               scale: float, mul_prev: int, mul_cur: int, sb):
+    """Scaled token embedding plus a hashed embedding of the (previous, current) token pair: row
+    ``(prev*mul_prev + cur*mul_cur) mod buckets`` of ``pair_table`` ``[buckets + 1, W]``; a sequence's first token
+    takes the extra last row.  ``prev`` (int32 ``[slots]``) carries each sequence's last token from step to step
+    and is updated in place.  Returns ``(x float [T, W], x in the table's dtype)``."""
+    from . import reference as ref
+    from ._native import native_seq, use_seq
+    if use_seq(table):
+        return tuple(native_seq().embed_pair(tokens.reshape(-1).long().contiguous(), table, pair_table, prev, scale,
+                                             mul_prev, mul_cur, sb.desc, sb.live))
+    return ref.embed_pair(tokens, table, pair_table, prev, scale, mul_prev, mul_cur, sb)

@@ -135,3 +135,80 @@ def moe_combine(ys: torch.Tensor, d: Dispatch, w: torch.Tensor, base: torch.Tens
     g = ys.index_select(0, d.pos_of.long()).view(T, d.k, -1)
     out = (g * w.to(ys.dtype).unsqueeze(-1)).sum(1)
     return out if base is None else out + base
+
+
+# ------------------------------------------------------------------ serving: grouped routing, identity experts
+def route_grouped(logits: torch.Tensor, correction: torch.Tensor | None, top: int, groups: int = 1, keep: int = 1,
+                  scale: float = 1.0):
+    """Float router logits ``[T, n]`` -> ``(expert ids int32 [T, top], weights float [T, top])``.  Scores are the
+    softmax over all ``n`` outputs; the choice is made on ``score + correction``, restricted to the ``keep`` best of
+    ``groups`` equal runs of neighbouring outputs (a run's rank is its largest choice value); the weights are the
+    plain scores times ``scale``, not renormalised."""
+    from . import reference as ref
+    from ._native import native_seq, use_seq
+    if use_seq(logits):
+        idx, w = native_seq().route_grouped(logits.contiguous(), correction, top, groups, keep, scale)
+        return idx, w
+    return ref.route_grouped(logits, correction, top, groups, keep, scale)
+
+
+def route_tokens(h: torch.Tensor, router: torch.Tensor, correction: torch.Tensor | None, top: int, groups: int = 1,
+                 keep: int = 1, scale: float = 1.0):
+    """:func:`route_grouped` on the logits ``h @ router^T`` (``router`` float ``[n, W]``; the products accumulate in
+    float whatever ``h``'s dtype).  On the GPU product and routing are one kernel."""
+    from ._native import native_seq, use_seq
+    if use_seq(h):
+        idx, w = native_seq().route_fused(h, router, correction, top, groups, keep, scale)
+        return idx, w
+    return route_grouped(h.float() @ router.t(), correction, top, groups, keep, scale)
+
+
+PAD_ROWS = 128      # sorted path: an expert's products run over a multiple of this many rows (0: exactly its rows)
+
+
+def moe_glu_experts(h: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.Tensor, idx: torch.Tensor,
+                    weights: torch.Tensor, limit: float, shared: torch.Tensor | None = None,
+                    few_tokens: bool = False) -> torch.Tensor:
+    """Weighted sum of the chosen clipped-GLU experts' outputs, float ``[T, W]``.  ``w_gate_up`` ``[E, 2, F, W]``,
+    ``w_down`` ``[E, W, F]``; ids ``>= E`` are identity experts (their output is ``h``); ``shared`` ``[T, W]`` is
+    added.  ``few_tokens`` (decode steps, captured graphs): every (token, expert) pair streams its expert's rows in
+    two kernels with no sort and no host round trip.  Otherwise rows are sorted by expert, every expert runs one
+    vendor matrix product pair over its run of rows (one host read of the run lengths; long runs are rounded up to a
+    multiple of ``PAD_ROWS`` rows), and a kernel combines."""
+    from . import reference as ref
+    from ._native import native_seq, use_seq
+    from .activation import clipped_glu
+    T, W = h.shape
+    E, _, F_, _ = w_gate_up.shape
+    top = idx.shape[1]
+    if use_seq(h) and few_tokens:
+        return native_seq().moe_pairs(h.contiguous(), w_gate_up, w_down, idx, weights, shared, limit)
+    flat = idx.reshape(-1).long()
+    order = torch.sort(flat, stable=True).indices
+    counts = torch.bincount(flat, minlength=E).tolist()[:E]
+    rows = sum(counts)
+    # every expert's products run over its rows rounded up to a multiple of PAD_ROWS (the surplus rows belong to the
+    # next experts, whose own products overwrite them afterwards, or to the zero tail): a stream of prompts then
+    # meets few distinct GEMM shapes instead of a new one per expert and prompt
+    pad = PAD_ROWS if rows >= 4 * PAD_ROWS else 0
+    xs = h.new_empty(rows + pad, W)
+    torch.index_select(h, 0, (order // top)[:rows], out=xs[:rows])
+    xs[rows:].zero_()
+    ys = torch.empty(rows + pad, W, dtype=h.dtype, device=h.device)
+    a = 0
+    for e, n in enumerate(counts):
+        if n:
+            m = min(-(-n // pad) * pad, rows + pad - a) if pad else n
+            z = xs[a:a + m] @ w_gate_up[e].reshape(2 * F_, W).t()
+            torch.mm(clipped_glu(z, limit), w_down[e].t(), out=ys[a:a + m])
+            a += n
+    pos = torch.empty_like(order)
+    pos[order] = torch.arange(order.numel(), device=order.device)
+    if use_seq(h):
+        return native_seq().moe_combine_sorted(ys, pos.contiguous(), idx, weights, h.contiguous(), shared, E)
+    pos = pos.view(T, top)
+    own = idx.long() >= E
+    picked = torch.where(own[..., None], h.float()[:, None, :], ys.float()[pos.clamp(max=max(rows - 1, 0))]
+                         if rows else h.float()[:, None, :].expand(T, top, W))
+    out = (picked * weights[..., None]).sum(1)
+    return out if shared is None else out + shared.float()

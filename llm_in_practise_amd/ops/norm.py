@@ -155,3 +155,30 @@ def head_norm_gate(o: torch.Tensor, weight: torch.Tensor, gate_pre: torch.Tensor
     if den is not None:
         o = o / (torch.maximum(den.abs(), floor) + 1e-6)[..., None]
     return ref.head_norm_gate(o, weight, gate_pre, eps)
+
+
+def scaled_postnorm(x: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, alpha: float, eps: float,
+                    dtype: torch.dtype) -> torch.Tensor:
+    """The sublayer exit of a post-normed block, in place on the float residual: ``x <- rmsnorm(alpha*x + y) * weight``
+    (``y`` float or the activation dtype); returns ``x`` in the activation ``dtype`` for the next matrix product."""
+    from ._native import native_seq, use_seq
+    if use_seq(x):
+        return native_seq().scaled_postnorm(x, y, weight, alpha, eps, dtype == torch.bfloat16)
+    return ref.scaled_postnorm(x, y, weight, alpha, eps, dtype)
+
+
+def rms_norm_act(u: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    """RMS norm of activation rows ``[T, n]`` (a column slice of a wider matrix is fine), statistics in float."""
+    from ._native import native_seq, use_seq
+    if use_seq(u):
+        return native_seq().rms_act(u, weight, eps)
+    return ref.rms_act(u, weight, eps)
+
+
+def gate_group_norm(y: torch.Tensor, z: torch.Tensor, weight: torch.Tensor, parts: int, eps: float) -> torch.Tensor:
+    """Gate, then norm: ``v = y * silu(z)`` (``y`` float ``[T, n]``, ``z`` activation dtype), each of ``parts`` equal
+    runs of ``v`` divided by its own root mean square, times ``weight``; returns the activation dtype."""
+    from ._native import native_seq, use_seq
+    if use_seq(y):
+        return native_seq().gate_group_norm(y, z, weight, parts, eps)
+    return ref.gate_group_norm(y, z, weight, parts, eps)

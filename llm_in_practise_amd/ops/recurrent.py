@@ -2,8 +2,9 @@
 
 * :func:`mlstm_scan` — the mLSTM cell of xLSTM with exponential gating stabilised by a running maximum.
 * :func:`gated_delta_scan` — the delta rule with a per-key-channel decay (erase, then write the prediction error).
+* :func:`ssd_scan` — a selective state space in its state-space-duality form (scalar decay and step size per head).
 
-Both keep ``S`` as ``[slots, H, dv, dk]`` float (one column of the ``[dk, dv]`` matrix contiguous), read
+All keep ``S`` as ``[slots, H, dv, dk]`` float (one column of the ``[dk, dv]`` matrix contiguous), read
 and write it in place, and treat a sequence that starts at position 0 as starting from zero state.  The same kernel
 serves prefill (a scan over the step's tokens with the state in registers) and decode (one token: load, update,
 store).  HIP kernels: csrc/kernels/seq/seq_scan.hip; the CPU path is ops/reference.py.
@@ -44,3 +45,13 @@ def gated_delta_scan(q, k, v, g, beta_pre, S, heads: int, kv_heads: int, sb):
         return native_seq().delta_scan(q, k, v, g.contiguous(), beta_pre.contiguous(), S, heads, kv_heads, sb.desc,
                                        sb.live)
     return ref.delta_scan(q, k, v, g, beta_pre, S, heads, kv_heads, sb)
+
+
+def ssd_scan(c, b, x, dt_raw, dt_bias, a_log, d_skip, S, heads: int, groups: int, sb):
+    """Selective state space, one scalar decay per head: ``dt = softplus(dt_raw + dt_bias)``,
+    ``S <- exp(-exp(a_log) dt) S + b (dt x)^T``, ``y = S^T c + d_skip x``.  ``c, b`` ``[T, G*N]`` and ``x`` ``[T, H*P]``
+    in the activation dtype, ``dt_raw`` ``[T, H]`` (a column slice is fine); head ``h`` reads group ``h // (H/G)``;
+    ``S`` float ``[slots, H, P, N]``.  Step sizes, decays and the state are float.  Returns float ``[T, H*P]``."""
+    if use_seq(c):
+        return native_seq().ssd_scan(c, b, x, dt_raw, dt_bias, a_log, d_skip, S, heads, groups, sb.desc, sb.live)
+    return ref.ssd_scan(c, b, x, dt_raw, dt_bias, a_log, d_skip, S, heads, groups, sb)

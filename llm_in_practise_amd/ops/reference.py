@@ -195,7 +195,7 @@ def decay_gate(pre, bias, a_log, dk: int):
     return torch.exp(-torch.exp(a_log)[None, :, None] * dt).reshape(T, HD)
 
 
-def short_conv(u, w, state, segs, seg_w, seg_scale, sb, eps: float, out_f32: bool):
+def short_conv(u, w, state, segs, seg_w, seg_scale, sb, eps: float, out_f32: bool, bias=None):
     T, C = u.shape
     taps = w.shape[1]
     off, slots, pos0 = sb.host()
@@ -211,6 +211,8 @@ def short_conv(u, w, state, segs, seg_w, seg_scale, sb, eps: float, out_f32: boo
             ext = u[a:e].float()
         win = ext.unfold(0, taps, 1)                       # [len, C, taps]
         y[a:e] = (win * w[None]).sum(-1)
+    if bias is not None:
+        y = y + bias
     out = torch.empty_like(y)
     for (c0, nh, hw, mode), sw, sc in zip(segs, seg_w, seg_scale):
         v = y[:, c0:c0 + nh * hw].view(T, nh, hw)
@@ -290,3 +292,124 @@ def talk_attention(q, kc, vc, talk, gate, H: int, G: int, scale: float, sb):
         w = torch.einsum("hg,gtl->htl", talk, w)
         out[a:e] = torch.einsum("htl,lhd->thd", w, vv).reshape(e - a, H * dv)
     return (out * torch.sigmoid(gate.float())).to(q.dtype)
+
+
+# ---- post-norm hybrid layers (state-space mixers, latent attention, routed experts)
+def embed_pair(tok, table, pair, prev, scale: float, mul_prev: int, mul_cur: int, sb):
+    tok = tok.reshape(-1).long()
+    x = table[tok].float() * scale
+    if pair is not None:
+        buckets = pair.shape[0] - 1
+        off, slots, pos0 = sb.host()
+        rows = torch.empty_like(tok)
+        for b, slot in enumerate(slots):
+            a, e = off[b], off[b + 1]
+            before = torch.cat([prev[slot].long().reshape(1), tok[a:e - 1]])
+            rows[a:e] = (before * mul_prev + tok[a:e] * mul_cur) % buckets
+            if pos0[b] == 0:
+                rows[a] = buckets
+            if sb.is_live(b):
+                prev[slot] = tok[e - 1].to(prev.dtype)
+        x = x + pair[rows].float()
+    return x, x.to(table.dtype)
+
+
+def scaled_postnorm(x, y, w, alpha: float, eps: float, dtype):
+    x.copy_(_unit_rms(alpha * x + y.float(), eps) * w)
+    return x.to(dtype)
+
+
+def rms_act(u, w, eps: float):
+    return (_unit_rms(u.float(), eps) * w).to(u.dtype)
+
+
+def gate_group_norm(y, z, w, parts: int, eps: float):
+    T, n = y.shape
+    v = y * F.silu(z.float())
+    return (_unit_rms(v.view(T, parts, n // parts), eps).reshape(T, n) * w).to(z.dtype)
+
+
+def ssd_scan(q, k, v, dtraw, dt_bias, a_log, dskip, S, H: int, G: int, sb):
+    T = q.shape[0]
+    dk, dv = q.shape[1] // G, v.shape[1] // H
+    rep = H // G
+    qf = q.float().view(T, G, dk).repeat_interleave(rep, 1)
+    kf = k.float().view(T, G, dk).repeat_interleave(rep, 1)
+    vf = v.float().view(T, H, dv)
+    dt = F.softplus(dtraw.float() + dt_bias)
+    decay = torch.exp(-torch.exp(a_log) * dt)
+    out = torch.empty(T, H, dv, dtype=torch.float32, device=q.device)
+    off, slots, pos0 = sb.host()
+    for b, slot in enumerate(slots):
+        if not sb.is_live(b):
+            continue
+        s = torch.zeros_like(S[slot]) if pos0[b] == 0 else S[slot].clone()   # [H, dv, dk]
+        for t in range(off[b], off[b + 1]):
+            s = decay[t][:, None, None] * s + (dt[t][:, None] * vf[t])[:, :, None] * kf[t][:, None, :]
+            out[t] = (s * qf[t][:, None, :]).sum(-1) + dskip[:, None] * vf[t]
+        S[slot] = s
+    return out.reshape(T, H * dv)
+
+
+def rotate_pairs(v, pos, inv_freq, dims: int):
+    """v [T, ..., d] float: neighbours (2i, 2i+1) below ``dims`` turn by pos * inv_freq[i]."""
+    if dims == 0:
+        return v
+    ang = pos.float().reshape(-1, *([1] * (v.dim() - 1))) * inv_freq[: dims // 2].float()
+    c, s = torch.cos(ang), torch.sin(ang)
+    a, b = v[..., 0:dims:2], v[..., 1:dims:2]
+    out = v.clone()
+    out[..., 0:dims:2] = a * c - b * s
+    out[..., 1:dims:2] = b * c + a * s
+    return out
+
+
+def latent_kv_store(u, w, inv_freq, cache, dims: int, eps: float, sb):
+    R = w.numel()
+    c = _unit_rms(u[:, :R].float(), eps) * w
+    kr = rotate_pairs(u[:, R:].float(), sb.desc[4], inv_freq, dims)
+    cache.view(-1, cache.shape[2]).index_copy_(0, sb.cache_idx, torch.cat([c, kr], 1).to(cache.dtype))
+
+
+def latent_attention(qa, q, cache, gate, inv_freq, H: int, dn: int, dims: int, scale: float, sb):
+    T, R = q.shape[0], qa.shape[2]
+    dr = q.shape[1] // H - dn
+    qr = rotate_pairs(q.float().view(T, H, dn + dr)[..., dn:], sb.desc[4], inv_freq, dims)
+    Q = torch.cat([qa.transpose(0, 1).float(), qr], -1).to(q.dtype).float()       # [T, H, R + dr]
+    out = torch.empty(T, H, R, dtype=torch.float32, device=q.device)
+    off, slots, pos0 = sb.host()
+    for b, slot in enumerate(slots):
+        a, e = off[b], off[b + 1]
+        L = pos0[b] + e - a
+        rows = cache[slot, :L].float()
+        sc = torch.einsum("thd,ld->htl", Q[a:e], rows) * scale
+        vis = torch.arange(L, device=q.device)[None, :] <= (pos0[b] + torch.arange(e - a, device=q.device))[:, None]
+        w = torch.softmax(sc.masked_fill(~vis[None], float("-inf")), -1)
+        out[a:e] = torch.einsum("htl,lr->thr", w, rows[:, :R])
+    if gate is not None:
+        out = out * torch.sigmoid(gate.float())[..., None]
+    return out.to(q.dtype)
+
+
+def route_grouped(z, corr, top: int, groups: int, keep: int, scale: float):
+    T, n = z.shape
+    s = torch.softmax(z.float(), -1)
+    ch = s + corr if corr is not None else s.clone()
+    if groups > 1 and keep < groups:
+        best = ch.view(T, groups, n // groups).max(-1).values
+        kept = torch.zeros(T, groups, dtype=torch.bool, device=z.device)
+        kept.scatter_(1, best.topk(keep, -1).indices, True)
+        ch = ch.masked_fill(~kept.repeat_interleave(n // groups, 1), float("-inf"))
+    idx = ch.topk(top, -1).indices
+    return idx.int(), s.gather(1, idx) * scale
+
+
+def clipped_glu(z, limit: float):
+    F_ = z.shape[-1] // 2
+    g = z[..., :F_].float().clamp(max=limit)
+    u = z[..., F_:].float().clamp(-limit, limit)
+    return (g * torch.sigmoid(1.702 * g) * (u + 1.0)).to(z.dtype)
+
+
+def gelu_tanh(z):
+    return F.gelu(z.float(), approximate="tanh").to(z.dtype)
