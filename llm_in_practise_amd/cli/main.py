@@ -293,7 +293,7 @@ def _load_for_inference(path, adapter=None, device=None, quant=None, fuse=True, 
             from ..quant.io import load_quantized
             m = load_quantized(path, dev)
         else:
-            from ..models.registry import load_causal_lm      # the class config.json names (Qwen3/Qwen2, Mobupel)
+            from ..models.registry import load_causal_lm      # the class config.json names (Qwen3/Qwen2, Mobupel, Dogudra)
             bnb = BitsAndBytesConfig(load_in_4bit=True) if quant == "nf4" else None
             m = load_causal_lm(path, dtype=torch.bfloat16, device=dev, quantization_config=bnb)
     if adapter:

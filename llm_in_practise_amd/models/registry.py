@@ -20,9 +20,15 @@ def _mobupel():
     return MobupelForCausalLM
 
 
+def _dogudra():
+    from .dogudra import DogudraForCausalLM
+    return DogudraForCausalLM
+
+
 REGISTRY = {
     "qwen3": _qwen, "qwen2": _qwen, "qwen3forcausallm": _qwen, "qwen2forcausallm": _qwen,
     "mobupel": _mobupel, "mobupelforcausallm": _mobupel,
+    "dogudra": _dogudra, "dogudraforcausallm": _dogudra,
 }
 
 
